@@ -1,0 +1,177 @@
+/*
+ * libmagi_attn: C-ABI for the MAGI-1 DiT attention hot path on MI355X (gfx950).
+ *
+ * Every function returns 0 on success or a negative MAGI_E* code and never throws or
+ * aborts; magi_last_error() returns a thread-local message for the last failure.  The
+ * caller owns every device buffer; except where a function says otherwise the library
+ * allocates no device memory, performs no host synchronisation and launches on the
+ * stream it is given (hipStream_t passed as void*; NULL = the default stream).
+ *
+ * The reference has no FFI of its own: it binds four Python callables from third-party
+ * CUDA packages.  Each entry point below names the reference call site it stands in for
+ * (paths relative to the reference checkout).
+ */
+#ifndef MAGI_ATTN_H
+#define MAGI_ATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MAGI_OK 0
+#define MAGI_EINVAL (-22)   /* bad argument (shape, stride, alignment, dtype) */
+#define MAGI_ENOSYS (-38)   /* configuration not implemented (e.g. head_dim != 128) */
+#define MAGI_EHIP (-5)      /* a HIP runtime call failed; see magi_last_error() */
+
+/* element types of q / k / v */
+#define MAGI_DTYPE_BF16 0
+#define MAGI_DTYPE_FP8_E4M3 1 /* OCP e4m3fn with per-(chunk, head) fp32 scales */
+
+/* how q_ranges / k_ranges are encoded */
+#define MAGI_RANGES_PAIRS 0 /* int32 [n, 2]: range i = [r[2i], r[2i+1])          */
+#define MAGI_RANGES_CU 1    /* int32 [n + 1] cumulative: range i = [r[i], r[i+1]) */
+
+/* QK-norm kinds of the prologue */
+#define MAGI_NORM_LAYERNORM_1P 0 /* (x-mean)/sqrt(var+eps) * (gamma+1) + beta */
+#define MAGI_NORM_RMSNORM_1P 1   /* x/sqrt(mean(x^2)+eps) * (gamma+1)          */
+#define MAGI_NORM_NONE 2
+
+int magi_version(void);
+const char* magi_last_error(void);
+
+/*
+ * Range attention forward (bf16 or fp8-e4m3 inputs, fp32 softmax, bf16 output).
+ *
+ *   for each i < n_ranges:
+ *     out[q_range_i, h, :] = softmax(q[q_range_i, h] . k[k_range_i, h / (Hq/Hkv)]^T * scale) v[k_range_i, h / (Hq/Hkv)]
+ *
+ * with no mask inside a rectangle.  q ranges must be disjoint; rows of `out` that no range
+ * covers are left untouched; a range with no keys writes zeros (and lse = -inf).
+ *
+ * Stands in for
+ *   flex_flash_attn_func(q, k, v, q_ranges, k_ranges, max_seqlen_q, max_seqlen_k, softmax_scale, ...)
+ *       inference/model/dit/dit_module.py:1032-1043, 1074-1085, 1111-1122
+ *   flash_attn_func(q, k, v)                 inference/model/dit/dit_module.py:1062, 1090-1095  (one range)
+ *   flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, ...)   dit_module.py:1124-1133 (MAGI_RANGES_CU)
+ *
+ * q   [total_q, Hq, D]   element strides q_stride_t (token), q_stride_h (head); D contiguous
+ * k,v [total_k, Hkv, D]  element strides k_stride_t/h and v_stride_t/h.  K and V may alias one
+ *                        interleaved KV-cache allocation [T, Hkv, 2D] (k = cache, v = cache + D):
+ *                        the cache is read in place, which removes the prefix slice / cat /
+ *                        contiguous copies of dit_module.py:915, 931, 945-946, 1027-1029.
+ * k2,v2                  optional second segment (NULL to disable): key rows >= k_split are read
+ *                        from k2/v2 at row (index - k_split) with the same strides.  This is how
+ *                        "attend to the new KV without persisting it" (update_kv_cache == False,
+ *                        dit_module.py:918-931) works without a copy.
+ * out [total_q, Hq, D]   bf16, strides o_stride_t / o_stride_h
+ * lse                    optional fp32 [Hq, total_q] (NULL to skip)
+ * q_ranges, k_ranges     DEVICE int32 arrays, encoding per ranges_mode; clamped to
+ *                        [0,total_q] / [0,total_k] in the kernel
+ * max_seqlen_q           upper bound of any q range length (host int; sizes the grid)
+ * q_scale,k_scale,v_scale  fp8 only: DEVICE fp32 [n_scale_chunks, H] with the scale of token t
+ *                        at [t / scale_chunk_tokens, h]; NULL for bf16
+ * softmax_scale          <= 0 selects D^-0.5
+ */
+typedef struct magi_attn_args {
+  const void* q;
+  const void* k;
+  const void* v;
+  const void* k2;
+  const void* v2;
+  void* out;
+  float* lse;
+  const int32_t* q_ranges;
+  const int32_t* k_ranges;
+  const float* q_scale;
+  const float* k_scale;
+  const float* v_scale;
+  int64_t q_stride_t, q_stride_h;
+  int64_t k_stride_t, k_stride_h;
+  int64_t v_stride_t, v_stride_h;
+  int64_t o_stride_t, o_stride_h;
+  int32_t total_q, total_k, k_split;
+  int32_t n_ranges, ranges_mode;
+  int32_t max_seqlen_q, max_seqlen_k;
+  int32_t Hq, Hkv, D;
+  int32_t dtype;
+  int32_t scale_chunk_tokens;
+  float softmax_scale;
+  int32_t reserved;
+} magi_attn_args;
+
+int magi_attn_fwd(const magi_attn_args* args, void* stream);
+
+/*
+ * Fused QK-norm + partial non-interleaved rotary + bf16 cast + KV-cache write, one pass.
+ *
+ * Stands in for get_q / get_k / get_v / get_kv after the linear layers
+ * (inference/model/dit/dit_module.py:953-996: .float(), FusedLayerNorm :323-357, transpose,
+ * flash_attn.layers.rotary.apply_rotary_emb :961/:978, .to(bf16), rearrange, cat) and for the
+ * cache append of _full_adjust_key_and_value (dit_module.py:918-929).
+ *
+ * q_raw [S, Hq*D], k_raw / v_raw [S, Hkv*D]  bf16, token strides in elements
+ * rope  [S, 2*R2] fp32, sin in the first R2 columns, cos in the last R2 (dit_module.py:770, 1147);
+ *       rotary_dim = 2*R2 <= D; NULL disables rotary
+ * gq,bq,gk,bk  fp32 [D] norm parameters (gamma stored zero-centred); b* may be NULL
+ * q_out [S, Hq, D] bf16 contiguous (or fp8 with q_scale_out, see below)
+ * kv_out  row 0 of the destination for the first n_cache_rows tokens: [*, Hkv, 2D] with token
+ *         stride kv_stride_t; K goes to [..., 0:D], V to [..., D:2D]
+ * kv_tail destination of tokens >= n_cache_rows (same layout, row index t - n_cache_rows); may be
+ *         NULL when n_cache_rows == S
+ */
+typedef struct magi_prologue_args {
+  const void* q_raw;
+  const void* k_raw;
+  const void* v_raw;
+  const float* rope;
+  const float* gq;
+  const float* bq;
+  const float* gk;
+  const float* bk;
+  void* q_out;
+  void* kv_out;
+  void* kv_tail;
+  int64_t q_raw_stride_t, k_raw_stride_t, v_raw_stride_t;
+  int64_t kv_stride_t, kv_tail_stride_t;
+  int32_t S, n_cache_rows;
+  int32_t Hq, Hkv, D, R2;
+  int32_t norm_kind;
+  float eps;
+} magi_prologue_args;
+
+int magi_qk_prologue(const magi_prologue_args* args, void* stream);
+
+/*
+ * Per-head norm only (no rotary, no cache): x [S, H, D] bf16 -> y [S, H, D] bf16, computed in the
+ * precision the reference uses for the cross-attention norms (bf16 in, fp32 statistics, bf16 out).
+ * Stands in for q_layernorm_xattn / k_layernorm_xattn in get_xqkv (dit_module.py:1008, 1020).
+ * x token stride / head stride in elements (K of the interleaved xattn KV projection has
+ * head stride 2D); y is contiguous.
+ */
+int magi_head_norm(const void* x, int64_t x_stride_t, int64_t x_stride_h, const float* gamma, const float* beta,
+                   void* y, int32_t S, int32_t H, int32_t D, int32_t norm_kind, float eps, void* stream);
+
+/*
+ * Non-interleaved rotary on the first 2*R2 features, any float dtype handled as fp32 or bf16.
+ * Stands in for flash_attn.layers.rotary.apply_rotary_emb(x, cos, sin) (dit_module.py:961, 978).
+ * x, y [B, S, H, D] contiguous; cos, sin [S, R2] fp32; is_bf16 selects the element type of x / y.
+ */
+int magi_apply_rotary(const void* x, const float* cos, const float* sin, void* y, int32_t B, int32_t S, int32_t H,
+                      int32_t D, int32_t R2, int32_t is_bf16, void* stream);
+
+/*
+ * Per-(chunk, head) absmax scales and OCP e4m3fn quantisation for the fp8 attention path:
+ * scale[c, h] = max(absmax over tokens of chunk c and D, tiny) / 448;  y = sat_e4m3(x / scale).
+ * The quantiser follows the reference's only fp8 convention, div_clamp_to
+ * (dit_module.py:364-384: clamp to +-448, saturating e4m3fn), without its bf16 intermediate.
+ * x [T, H, D] bf16 with strides; y [T, H, D] fp8 contiguous; scales fp32 [ceil(T/chunk_tokens), H].
+ */
+int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, float* scales, int32_t T,
+                      int32_t H, int32_t D, int32_t chunk_tokens, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MAGI_ATTN_H */

@@ -1,0 +1,217 @@
+// C-ABI layer of libmagi_attn: argument validation, error reporting, kernel dispatch.
+#include <hip/hip_runtime.h>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "kernels.h"
+#include "magi_attn.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int hip_fail(hipError_t e, const char* what) {
+  return fail(MAGI_EHIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+int magi_version(void) { return 100; }
+
+const char* magi_last_error(void) { return g_err; }
+
+int magi_attn_fwd(const magi_attn_args* p, void* stream) {
+  if (!p) return fail(MAGI_EINVAL, "magi_attn_fwd: args is NULL");
+  if (p->D != 128) return fail(MAGI_ENOSYS, "magi_attn_fwd: head_dim %d not implemented (128 only)", p->D);
+  if (p->dtype != MAGI_DTYPE_BF16 && p->dtype != MAGI_DTYPE_FP8_E4M3)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: unknown dtype %d", p->dtype);
+  if (p->Hq <= 0 || p->Hkv <= 0 || p->Hq % p->Hkv != 0)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: Hq=%d must be a positive multiple of Hkv=%d", p->Hq, p->Hkv);
+  if (p->total_q < 0 || p->total_k < 0 || p->n_ranges < 0 || p->max_seqlen_q < 0)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: negative size");
+  if (p->ranges_mode != MAGI_RANGES_PAIRS && p->ranges_mode != MAGI_RANGES_CU)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: unknown ranges_mode %d", p->ranges_mode);
+  if (p->n_ranges == 0 || p->total_q == 0 || p->max_seqlen_q == 0) return MAGI_OK;
+  if (!p->q || !p->out || !p->q_ranges || !p->k_ranges) return fail(MAGI_EINVAL, "magi_attn_fwd: NULL q/out/ranges");
+  if (p->total_k > 0 && (!p->k || !p->v)) return fail(MAGI_EINVAL, "magi_attn_fwd: NULL k/v with total_k > 0");
+  const int esz = p->dtype == MAGI_DTYPE_BF16 ? 2 : 1;
+  const int64_t row_elems = 16 / esz;  // 16-byte vectors
+  if (p->q_stride_h % row_elems || p->q_stride_t % row_elems || p->k_stride_h % row_elems ||
+      p->k_stride_t % row_elems || p->v_stride_h % row_elems || p->v_stride_t % row_elems || p->o_stride_h % 8 ||
+      p->o_stride_t % 8)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: strides must keep rows 16-byte aligned");
+  if (!aligned16(p->q) || !aligned16(p->k) || !aligned16(p->v) || !aligned16(p->out) || !aligned16(p->k2) ||
+      !aligned16(p->v2))
+    return fail(MAGI_EINVAL, "magi_attn_fwd: q/k/v/out must be 16-byte aligned");
+  if (p->q_stride_h < p->D || p->k_stride_h < p->D || p->v_stride_h < p->D || p->o_stride_h < p->D)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: head stride smaller than head_dim");
+  int k_split = p->total_k;
+  if (p->k2 || p->v2) {
+    if (!p->k2 || !p->v2) return fail(MAGI_EINVAL, "magi_attn_fwd: k2 and v2 must be given together");
+    if (p->k_split < 0 || p->k_split > p->total_k)
+      return fail(MAGI_EINVAL, "magi_attn_fwd: k_split %d outside [0, total_k=%d]", p->k_split, p->total_k);
+    k_split = p->k_split;
+  }
+  if (p->dtype == MAGI_DTYPE_FP8_E4M3) {
+    if (!p->q_scale || !p->k_scale || !p->v_scale || p->scale_chunk_tokens <= 0)
+      return fail(MAGI_EINVAL, "magi_attn_fwd: fp8 needs q/k/v scales and scale_chunk_tokens > 0");
+  }
+
+  magi::AttnKernArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.q = static_cast<const char*>(p->q);
+  a.k = static_cast<const char*>(p->k);
+  a.v = static_cast<const char*>(p->v);
+  a.k2 = static_cast<const char*>(p->k2);
+  a.v2 = static_cast<const char*>(p->v2);
+  a.out = static_cast<char*>(p->out);
+  a.lse = p->lse;
+  a.q_ranges = p->q_ranges;
+  a.k_ranges = p->k_ranges;
+  a.q_scale = p->q_scale;
+  a.k_scale = p->k_scale;
+  a.v_scale = p->v_scale;
+  a.qs_t = p->q_stride_t * esz;
+  a.qs_h = p->q_stride_h * esz;
+  a.ks_t = p->k_stride_t * esz;
+  a.ks_h = p->k_stride_h * esz;
+  a.vs_t = p->v_stride_t * esz;
+  a.vs_h = p->v_stride_h * esz;
+  a.os_t = p->o_stride_t * 2;
+  a.os_h = p->o_stride_h * 2;
+  a.total_q = p->total_q;
+  a.total_k = p->total_k;
+  a.k_split = k_split;
+  a.n_ranges = p->n_ranges;
+  a.ranges_mode = p->ranges_mode;
+  a.tiles_per_range = (p->max_seqlen_q + magi::kAttnBlockM - 1) / magi::kAttnBlockM;
+  a.Hq = p->Hq;
+  a.Hkv = p->Hkv;
+  a.G = p->Hq / p->Hkv;
+  a.scale_chunk_tokens = p->scale_chunk_tokens;
+  const double total = (double)p->Hq * p->n_ranges * a.tiles_per_range;
+  if (total > 2.0e9) return fail(MAGI_EINVAL, "magi_attn_fwd: grid too large (%.3g workgroups)", total);
+  a.total_wgs = (unsigned)total;
+  a.per_xcd = (a.total_wgs + 7u) / 8u;
+  const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 1.0f / std::sqrt((float)p->D);
+  a.scale_log2 = scale * 1.4426950408889634f;
+
+  hipError_t e = p->dtype == MAGI_DTYPE_BF16 ? magi::launch_attn_fwd_bf16(a, static_cast<hipStream_t>(stream))
+                                             : magi::launch_attn_fwd_fp8(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "magi_attn_fwd launch");
+  return MAGI_OK;
+}
+
+int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
+  if (!p) return fail(MAGI_EINVAL, "magi_qk_prologue: args is NULL");
+  if (p->D != 128) return fail(MAGI_ENOSYS, "magi_qk_prologue: head_dim %d not implemented (128 only)", p->D);
+  if (p->S < 0 || p->Hq < 0 || p->Hkv < 0) return fail(MAGI_EINVAL, "magi_qk_prologue: negative size");
+  if (p->S == 0 || p->Hq + p->Hkv == 0) return MAGI_OK;
+  if (p->R2 < 0 || p->R2 % 8 || 2 * p->R2 > p->D)
+    return fail(MAGI_EINVAL, "magi_qk_prologue: R2=%d must be a multiple of 8 with 2*R2 <= D", p->R2);
+  if (p->norm_kind < 0 || p->norm_kind > 2) return fail(MAGI_EINVAL, "magi_qk_prologue: norm_kind %d", p->norm_kind);
+  if (p->Hq > 0 && (!p->q_raw || !p->q_out)) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL q_raw/q_out");
+  if (p->Hkv > 0 && (!p->k_raw || !p->v_raw)) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL k_raw/v_raw");
+  if (p->n_cache_rows < 0 || p->n_cache_rows > p->S)
+    return fail(MAGI_EINVAL, "magi_qk_prologue: n_cache_rows %d outside [0, S=%d]", p->n_cache_rows, p->S);
+  if (p->Hkv > 0 && p->n_cache_rows > 0 && !p->kv_out) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL kv_out");
+  if (p->Hkv > 0 && p->n_cache_rows < p->S && !p->kv_tail)
+    return fail(MAGI_EINVAL, "magi_qk_prologue: kv_tail needed for rows >= n_cache_rows");
+  if (p->norm_kind != MAGI_NORM_NONE && ((p->Hq > 0 && !p->gq) || (p->Hkv > 0 && !p->gk)))
+    return fail(MAGI_EINVAL, "magi_qk_prologue: NULL gamma");
+  if (p->R2 > 0 && p->rope && (reinterpret_cast<uintptr_t>(p->rope) & 15u))
+    return fail(MAGI_EINVAL, "magi_qk_prologue: rope must be 16-byte aligned");
+  if (p->q_raw_stride_t % 8 || p->k_raw_stride_t % 8 || p->v_raw_stride_t % 8 || p->kv_stride_t % 8 ||
+      p->kv_tail_stride_t % 8)
+    return fail(MAGI_EINVAL, "magi_qk_prologue: strides must keep rows 16-byte aligned");
+  if (!aligned16(p->q_raw) || !aligned16(p->k_raw) || !aligned16(p->v_raw) || !aligned16(p->q_out) ||
+      !aligned16(p->kv_out) || !aligned16(p->kv_tail))
+    return fail(MAGI_EINVAL, "magi_qk_prologue: buffers must be 16-byte aligned");
+
+  magi::PrologueKernArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.q_raw = static_cast<const char*>(p->q_raw);
+  a.k_raw = static_cast<const char*>(p->k_raw);
+  a.v_raw = static_cast<const char*>(p->v_raw);
+  a.rope = p->R2 > 0 ? p->rope : nullptr;
+  a.gq = p->gq;
+  a.bq = p->bq;
+  a.gk = p->gk;
+  a.bk = p->bk;
+  a.q_out = static_cast<char*>(p->q_out);
+  a.kv_out = static_cast<char*>(p->kv_out);
+  a.kv_tail = static_cast<char*>(p->kv_tail);
+  a.q_raw_stride_t = p->q_raw_stride_t * 2;
+  a.k_raw_stride_t = p->k_raw_stride_t * 2;
+  a.v_raw_stride_t = p->v_raw_stride_t * 2;
+  a.kv_stride_t = p->kv_stride_t * 2;
+  a.kv_tail_stride_t = p->kv_tail_stride_t * 2;
+  a.S = p->S;
+  a.n_cache_rows = p->n_cache_rows;
+  a.Hq = p->Hq;
+  a.Hkv = p->Hkv;
+  a.R2 = a.rope ? p->R2 : 0;
+  a.norm_kind = p->norm_kind;
+  a.eps = p->eps;
+  hipError_t e = magi::launch_prologue(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "magi_qk_prologue launch");
+  return MAGI_OK;
+}
+
+int magi_head_norm(const void* x, int64_t x_stride_t, int64_t x_stride_h, const float* gamma, const float* beta,
+                   void* y, int32_t S, int32_t H, int32_t D, int32_t norm_kind, float eps, void* stream) {
+  if (D != 128) return fail(MAGI_ENOSYS, "magi_head_norm: head_dim %d not implemented (128 only)", D);
+  if (S < 0 || H < 0) return fail(MAGI_EINVAL, "magi_head_norm: negative size");
+  if (S == 0 || H == 0) return MAGI_OK;
+  if (!x || !y) return fail(MAGI_EINVAL, "magi_head_norm: NULL x/y");
+  if (norm_kind < 0 || norm_kind > 2) return fail(MAGI_EINVAL, "magi_head_norm: norm_kind %d", norm_kind);
+  if (norm_kind != MAGI_NORM_NONE && !gamma) return fail(MAGI_EINVAL, "magi_head_norm: NULL gamma");
+  if (x_stride_t % 8 || x_stride_h % 8 || !aligned16(x) || !aligned16(y))
+    return fail(MAGI_EINVAL, "magi_head_norm: rows must be 16-byte aligned");
+  hipError_t e = magi::launch_head_norm(static_cast<const char*>(x), x_stride_t * 2, x_stride_h * 2, gamma, beta,
+                                        static_cast<char*>(y), S, H, norm_kind, eps, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "magi_head_norm launch");
+  return MAGI_OK;
+}
+
+int magi_apply_rotary(const void* x, const float* cos, const float* sin, void* y, int32_t B, int32_t S, int32_t H,
+                      int32_t D, int32_t R2, int32_t is_bf16, void* stream) {
+  if (B < 0 || S < 0 || H < 0 || D <= 0 || D % 2) return fail(MAGI_EINVAL, "magi_apply_rotary: bad shape");
+  if (R2 < 0 || 2 * R2 > D) return fail(MAGI_EINVAL, "magi_apply_rotary: rotary_dim %d > head_dim %d", 2 * R2, D);
+  if ((long)B * S * H == 0) return MAGI_OK;
+  if (!x || !y || (R2 > 0 && (!cos || !sin))) return fail(MAGI_EINVAL, "magi_apply_rotary: NULL pointer");
+  hipError_t e = magi::launch_rotary(x, cos, sin, y, B, S, H, D, R2, is_bf16, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "magi_apply_rotary launch");
+  return MAGI_OK;
+}
+
+int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, float* scales, int32_t T,
+                      int32_t H, int32_t D, int32_t chunk_tokens, void* stream) {
+  if (D != 128) return fail(MAGI_ENOSYS, "magi_quantize_fp8: head_dim %d not implemented (128 only)", D);
+  if (T < 0 || H < 0 || chunk_tokens <= 0) return fail(MAGI_EINVAL, "magi_quantize_fp8: bad size");
+  if (T == 0 || H == 0) return MAGI_OK;
+  if (!x || !y || !scales) return fail(MAGI_EINVAL, "magi_quantize_fp8: NULL pointer");
+  if (x_stride_t % 8 || x_stride_h % 8 || !aligned16(x) || !aligned16(y))
+    return fail(MAGI_EINVAL, "magi_quantize_fp8: rows must be 16-byte aligned");
+  hipError_t e = magi::launch_quantize_fp8(static_cast<const char*>(x), x_stride_t * 2, x_stride_h * 2,
+                                           static_cast<char*>(y), scales, T, H, chunk_tokens,
+                                           static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "magi_quantize_fp8 launch");
+  return MAGI_OK;
+}
+
+}  // extern "C"

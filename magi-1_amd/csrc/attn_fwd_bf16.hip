@@ -1,0 +1,285 @@
+// Range attention forward, bf16 in / bf16 out, fp32 online softmax, for gfx950 (MI355X).
+//
+// One workgroup = 4 wavefronts = 128 query rows of one (range, q head); wave w owns rows
+// 32w..32w+31.  Key/value rows stream through LDS in tiles of 64, double buffered.
+//
+// The scores are computed transposed, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: the
+// accumulator layout then puts ONE query per lane column (lane % 32) and spreads the keys over
+// the registers, so row max / row sum are plain per-lane reductions plus one exchange between
+// the two half-waves, and the probabilities are already in the B-operand layout of the second
+// product O^T = V^T P^T.  V^T is fetched from the row-major V tile with the transposing LDS
+// read ds_read_b64_tr_b16.
+//
+// Work decomposition: blockIdx -> (kv head, range slot, q tile, q head within the GQA group),
+// laid out so that the workgroups an XCD receives (blockIdx % 8) share a KV head and walk the
+// same keys at about the same time (each XCD has its own L2).  Ranges are visited longest
+// first.  Fully masked key tiles never exist: a rectangle is walked from k_start to k_end only.
+#include "kernels.h"
+
+namespace magi {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
+
+constexpr int BM = kAttnBlockM;  // q rows per workgroup
+constexpr int BN = 64;           // keys per tile
+constexpr int ROW_BYTES = 256;   // D = 128 bf16
+constexpr int TILE_BYTES = BN * ROW_BYTES;
+constexpr int MAX_SORT = 256;
+
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
+  f32x2 x = {a, b};
+  bf16x2 r = __builtin_convertvector(x, bf16x2);
+  return __builtin_bit_cast(unsigned, r);
+}
+
+__device__ __forceinline__ void load_range(const int* r, int mode, int i, int total, int& s, int& e) {
+  if (mode == 0) {
+    s = r[2 * i];
+    e = r[2 * i + 1];
+  } else {
+    s = r[i];
+    e = r[i + 1];
+  }
+  s = max(0, min(s, total));
+  e = max(s, min(e, total));
+}
+
+__global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
+  __shared__ __attribute__((aligned(16))) unsigned char smem[2][2][TILE_BYTES];  // [buffer][K|V]
+  __shared__ int s_sel;
+
+  const int tid = threadIdx.x;
+  // ---- which piece of work is this workgroup? ----
+  const unsigned id = blockIdx.x;
+  const unsigned f = (id & 7u) * a.per_xcd + (id >> 3);
+  if (f >= a.total_wgs) return;
+  const unsigned per_range = (unsigned)a.tiles_per_range * (unsigned)a.G;
+  const unsigned per_kvh = (unsigned)a.n_ranges * per_range;
+  const unsigned kvh = f / per_kvh;
+  unsigned rem = f - kvh * per_kvh;
+  const unsigned rslot = rem / per_range;
+  rem -= rslot * per_range;
+  const unsigned tile = rem / (unsigned)a.G;
+  const unsigned hg = rem - tile * (unsigned)a.G;
+  const int h = (int)(kvh * a.G + hg);
+
+  // range with the rslot-th longest key span (ties by index)
+  int ridx;
+  if (a.n_ranges <= MAX_SORT) {
+    if (tid < a.n_ranges) {
+      int s, e;
+      load_range(a.k_ranges, a.ranges_mode, tid, a.total_k, s, e);
+      const int my = e - s;
+      int rank = 0;
+      for (int j = 0; j < a.n_ranges; ++j) {
+        int sj, ej;
+        load_range(a.k_ranges, a.ranges_mode, j, a.total_k, sj, ej);
+        const int lj = ej - sj;
+        rank += (lj > my) || (lj == my && j < tid);
+      }
+      if (rank == (int)rslot) s_sel = tid;
+    }
+    __syncthreads();
+    ridx = s_sel;
+  } else {
+    ridx = a.n_ranges - 1 - (int)rslot;
+  }
+  int qs, qe, ks, ke;
+  load_range(a.q_ranges, a.ranges_mode, ridx, a.total_q, qs, qe);
+  load_range(a.k_ranges, a.ranges_mode, ridx, a.total_k, ks, ke);
+  const int q0 = qs + (int)tile * BM;
+  if (q0 >= qe) return;
+
+  const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
+  const int q_row = q0 + 32 * w + i;
+  const bool row_ok = q_row < qe;
+
+  if (ke <= ks) {  // no keys: zeros, lse = -inf
+    if (row_ok) {
+      char* op = a.out + (long)q_row * a.os_t + (long)h * a.os_h + g * 128;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) *(u32x4*)(op + c * 16) = u32x4{0, 0, 0, 0};
+      if (a.lse && g == 0) a.lse[(long)h * a.total_q + q_row] = -__builtin_inff();
+    }
+    return;
+  }
+
+  // ---- Q fragments (B operand of S^T = K Q^T): lane (i, g) holds Q[row i][16kk + 8g .. +8] ----
+  bf16x8 qf[8];
+  {
+    const int qr = min(q_row, qe - 1);
+    const char* qp = a.q + (long)qr * a.qs_t + (long)h * a.qs_h + g * 16;
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 32);
+  }
+
+  // ---- K/V tile movers: thread owns 16-byte column chunk cc of rows r0 + 16j ----
+  const int cc = tid & 15, r0 = tid >> 4;
+  const long kcol = (long)kvh * a.ks_h + cc * 16;
+  const long vcol = (long)kvh * a.vs_h + cc * 16;
+  const int st_k = r0 * ROW_BYTES + ((cc ^ r0) << 4);               // K tile: chunk ^= row & 15
+  const int st_v = r0 * ROW_BYTES + ((cc ^ ((r0 & 3) << 2)) << 4);  // V tile: chunk ^= (row & 3) << 2
+  u32x4 kr[4], vr[4];
+
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int row = min(k0 + r0 + 16 * j, ke - 1);
+      const char* kb;
+      const char* vb;
+      if (row < a.k_split) {
+        kb = a.k + (long)row * a.ks_t;
+        vb = a.v + (long)row * a.vs_t;
+      } else {
+        kb = a.k2 + (long)(row - a.k_split) * a.ks_t;
+        vb = a.v2 + (long)(row - a.k_split) * a.vs_t;
+      }
+      kr[j] = *(const u32x4*)(kb + kcol);
+      vr[j] = *(const u32x4*)(vb + vcol);
+    }
+  };
+  auto stash = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      *LDS_PTR(u32x4, &smem[buf][0][st_k + j * 16 * ROW_BYTES]) = kr[j];
+      *LDS_PTR(u32x4, &smem[buf][1][st_v + j * 16 * ROW_BYTES]) = vr[j];
+    }
+  };
+
+  // ---- per-lane LDS read bases ----
+  // K as A operand: row = 32t + i, 16-byte chunk 2kk + g  ->  off = base_k ^ (kk << 5), + t * 32 rows
+  const int base_k = i * ROW_BYTES + (((i & 15) ^ g) << 4);
+  // V^T through the transposing read: 16-lane group q4 = l / 16 serves d block (q4 & 1), key group g;
+  // inside it lane 4r + c points at row r, 8-byte column unit c.
+  const int r4 = (l & 15) >> 2, c4 = l & 3, dblk = (l >> 4) & 1;
+  const int base_v = (4 * g + r4) * ROW_BYTES + ((r4 << 6) | (dblk << 5) | (c4 << 3));
+
+  f32x16 o_acc[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o_acc[mb][v] = 0.f;
+  float m_run = -__builtin_inff();  // running max of raw scores
+  float l_run = 0.f;                // this lane's share of the running sum
+  const float c = a.scale_log2;
+  const bool wave_on = (q0 + 32 * w) < qe;
+
+  const int n_tiles = (ke - ks + BN - 1) / BN;
+  fetch(ks);
+  for (int it = 0; it < n_tiles; ++it) {
+    const int buf = it & 1;
+    const int k0 = ks + it * BN;
+    stash(buf);
+    __syncthreads();
+    if (it + 1 < n_tiles) fetch(k0 + BN);
+    if (!wave_on) continue;
+
+    const unsigned char* Kt = &smem[buf][0][0];
+    const unsigned char* Vt = &smem[buf][1][0];
+
+    // S^T[key][q] for 64 keys x 32 queries
+    f32x16 s_acc[2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) s_acc[t][v] = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk) {
+        const bf16x8 ka = *LDS_PTR(const bf16x8, Kt + ((base_k ^ (kk << 5)) + t * 32 * ROW_BYTES));
+        s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s_acc[t], 0, 0, 0);
+      }
+    }
+    if (k0 + BN > ke) {  // ragged last tile: keys >= ke do not exist
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int key = k0 + 32 * t + 8 * (v >> 2) + 4 * g + (v & 3);
+          if (key >= ke) s_acc[t][v] = -__builtin_inff();
+        }
+    }
+    // online softmax: every value this lane holds belongs to query i
+    float mx = s_acc[0][0];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[t][v]);
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    const float m_new = fmaxf(m_run, mx);
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
+    const float mc = m_new * c;
+    m_run = m_new;
+    float psum = 0.f;
+    bf16x8 pb[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      u32x4 pk;
+#pragma unroll
+      for (int e = 0; e < 8; e += 2) {
+        const float p0 = __builtin_amdgcn_exp2f(s_acc[s >> 1][8 * (s & 1) + e] * c - mc);
+        const float p1 = __builtin_amdgcn_exp2f(s_acc[s >> 1][8 * (s & 1) + e + 1] * c - mc);
+        psum += p0 + p1;
+        pk[e >> 1] = pack_bf16x2(p0, p1);
+      }
+      pb[s] = __builtin_bit_cast(bf16x8, pk);
+    }
+    l_run = l_run * alpha + psum;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+
+    // O^T[d][q] += V^T[d][key] P^T[key][q]
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      const int bv = base_v ^ (mb << 6);
+#pragma unroll
+      for (int s = 0; s < 4; ++s) {
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * s) * ROW_BYTES)));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * s + 8) * ROW_BYTES)));
+        const s16x8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        o_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va), pb[s], o_acc[mb], 0, 0, 0);
+      }
+    }
+  }
+
+  if (!wave_on) return;
+  // ---- epilogue: normalise and store ----
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = 1.f / l_tot;
+  if (row_ok) {
+    char* op = a.out + (long)q_row * a.os_t + (long)h * a.os_h;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int d = 32 * mb + 8 * b + 4 * g;
+        u32x2 pk;
+        pk[0] = pack_bf16x2(o_acc[mb][4 * b + 0] * inv, o_acc[mb][4 * b + 1] * inv);
+        pk[1] = pack_bf16x2(o_acc[mb][4 * b + 2] * inv, o_acc[mb][4 * b + 3] * inv);
+        *(u32x2*)(op + d * 2) = pk;
+      }
+    if (a.lse && g == 0)
+      a.lse[(long)h * a.total_q + q_row] = (m_run * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+  }
+}
+
+}  // namespace
+
+hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
+  const unsigned grid = a.per_xcd * 8u;
+  hipLaunchKernelGGL(attn_fwd_bf16_kernel, dim3(grid), dim3(kAttnThreads), 0, stream, a);
+  return hipGetLastError();
+}
+
+}  // namespace magi

@@ -1,0 +1,66 @@
+// Internal launch interface between the C-ABI layer (api.cpp) and the HIP kernels.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace magi {
+
+// Arguments of the range-attention forward kernels.  All strides are in BYTES.
+struct AttnKernArgs {
+  const char* q;
+  const char* k;
+  const char* v;
+  const char* k2;
+  const char* v2;
+  char* out;
+  float* lse;
+  const int* q_ranges;
+  const int* k_ranges;
+  const float* q_scale;
+  const float* k_scale;
+  const float* v_scale;
+  long qs_t, qs_h, ks_t, ks_h, vs_t, vs_h, os_t, os_h;
+  int total_q, total_k, k_split;
+  int n_ranges, ranges_mode, tiles_per_range;
+  int Hq, Hkv, G;
+  int scale_chunk_tokens;
+  unsigned total_wgs, per_xcd;
+  float scale_log2;  // softmax_scale * log2(e)
+};
+
+// Q rows one workgroup covers (sizes the grid: tiles_per_range = ceil(max_seqlen_q / kAttnBlockM)).
+constexpr int kAttnBlockM = 128;
+constexpr int kAttnThreads = 256;
+
+hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream);
+hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream);
+
+struct PrologueKernArgs {
+  const char* q_raw;
+  const char* k_raw;
+  const char* v_raw;
+  const float* rope;
+  const float* gq;
+  const float* bq;
+  const float* gk;
+  const float* bk;
+  char* q_out;
+  char* kv_out;
+  char* kv_tail;
+  long q_raw_stride_t, k_raw_stride_t, v_raw_stride_t;  // bytes
+  long kv_stride_t, kv_tail_stride_t;                   // bytes
+  int S, n_cache_rows;
+  int Hq, Hkv, R2;
+  int norm_kind;
+  float eps;
+};
+hipError_t launch_prologue(const PrologueKernArgs& a, hipStream_t stream);
+
+hipError_t launch_head_norm(const char* x, long x_stride_t, long x_stride_h, const float* gamma, const float* beta,
+                            char* y, int S, int H, int norm_kind, float eps, hipStream_t stream);
+hipError_t launch_rotary(const void* x, const float* cos, const float* sin, void* y, int B, int S, int H, int D,
+                         int R2, int is_bf16, hipStream_t stream);
+hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
+                               int chunk_tokens, hipStream_t stream);
+
+}  // namespace magi

@@ -1,0 +1,249 @@
+// HBM-bound prologue kernels for gfx950: per-head QK norm + partial non-interleaved rotary +
+// bf16 cast + KV-cache write in one pass, plus the norm-only and rotary-only variants.
+//
+// Layout: 8 lanes serve one (token, head) row of D = 128 elements, 16 elements (two 16-byte
+// vectors) per lane, chosen so that a rotary pair (i, i + R2) lives in ONE lane: lanes
+// j < R2/8 hold x[8j..8j+7] and x[R2+8j..R2+8j+7], the remaining lanes hold the pass-through
+// tail in two consecutive vectors.  The rotation therefore needs no cross-lane traffic and the
+// norm statistics need three butterfly steps.  A wavefront covers 8 rows, a workgroup 32; all
+// global accesses are 16 bytes per lane and contiguous per row.
+#include "kernels.h"
+
+namespace magi {
+namespace {
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+constexpr int D = 128;
+constexpr int THREADS = 256;
+constexpr int GROUPS = THREADS / 8;  // rows in flight per workgroup
+constexpr int TOK_PER_BLOCK = 4;
+
+__device__ __forceinline__ void unpack8(const u32x4 v, float* f) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    f[2 * i] = __builtin_bit_cast(float, v[i] << 16);
+    f[2 * i + 1] = __builtin_bit_cast(float, v[i] & 0xffff0000u);
+  }
+}
+__device__ __forceinline__ unsigned pack2(float a, float b) {
+  f32x2 x = {a, b};
+  bf16x2 r = __builtin_convertvector(x, bf16x2);
+  return __builtin_bit_cast(unsigned, r);
+}
+__device__ __forceinline__ u32x4 pack8(const float* f) {
+  u32x4 v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v[i] = pack2(f[2 * i], f[2 * i + 1]);
+  return v;
+}
+__device__ __forceinline__ float group8_sum(float x) {
+  x += __shfl_xor(x, 1);
+  x += __shfl_xor(x, 2);
+  x += __shfl_xor(x, 4);
+  return x;
+}
+
+// Normalise the 16 values of this lane (8 lanes = one row of 128) in place.
+__device__ __forceinline__ void norm16(float* x, const float* gam, const float* bet, int ea, int eb, int kind, float eps,
+                                       bool has_beta) {
+  if (kind == 2) return;
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += x[i];
+  float mean = 0.f;
+  if (kind == 0) mean = group8_sum(s) * (1.f / D);
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const float d = x[i] - mean;
+    q += d * d;
+  }
+  const float rstd = __builtin_amdgcn_rsqf(group8_sum(q) * (1.f / D) + eps);
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int e = (i < 8) ? ea + i : eb + (i - 8);
+    float y = (x[i] - mean) * rstd * (gam[e] + 1.f);
+    if (kind == 0 && has_beta) y += bet[e];
+    x[i] = y;
+  }
+}
+
+__global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArgs a) {
+  __shared__ float s_par[4][D];  // gq, bq, gk, bk
+  const int tid = threadIdx.x;
+  for (int i = tid; i < 4 * D; i += THREADS) {
+    const int which = i / D, e = i % D;
+    const float* src = which == 0 ? a.gq : which == 1 ? a.bq : which == 2 ? a.gk : a.bk;
+    s_par[which][e] = src ? src[e] : 0.f;
+  }
+  __syncthreads();
+
+  const int j = tid & 7, grp = tid >> 3;
+  const int nr = a.R2 >> 3;  // lanes that hold rotary pairs
+  const bool rot_lane = j < nr;
+  const int ea = rot_lane ? 8 * j : 2 * a.R2 + 16 * (j - nr);  // first element of vector A
+  const int eb = rot_lane ? a.R2 + 8 * j : ea + 8;             // first element of vector B
+  const int U = a.Hq + 2 * a.Hkv;
+
+  for (int tt = 0; tt < TOK_PER_BLOCK; ++tt) {
+    const int s = blockIdx.x * TOK_PER_BLOCK + tt;
+    if (s >= a.S) break;
+    float sn[8], cs[8];
+    if (rot_lane && a.rope) {
+      const float* rp = a.rope + (long)s * (2 * a.R2);
+      const f32x4 s0 = *(const f32x4*)(rp + 8 * j), s1 = *(const f32x4*)(rp + 8 * j + 4);
+      const f32x4 c0 = *(const f32x4*)(rp + a.R2 + 8 * j), c1 = *(const f32x4*)(rp + a.R2 + 8 * j + 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        sn[i] = s0[i];
+        sn[4 + i] = s1[i];
+        cs[i] = c0[i];
+        cs[4 + i] = c1[i];
+      }
+    }
+    char* kvrow = (s < a.n_cache_rows) ? a.kv_out + (long)s * a.kv_stride_t
+                                       : a.kv_tail + (long)(s - a.n_cache_rows) * a.kv_tail_stride_t;
+    for (int u = grp; u < U; u += GROUPS) {
+      const char* src;
+      char* dst;
+      int kind;  // 0 = q, 1 = k, 2 = v
+      if (u < a.Hq) {
+        kind = 0;
+        src = a.q_raw + (long)s * a.q_raw_stride_t + (long)u * (D * 2);
+        dst = a.q_out + ((long)s * a.Hq + u) * (D * 2);
+      } else if (u < a.Hq + a.Hkv) {
+        kind = 1;
+        const int hh = u - a.Hq;
+        src = a.k_raw + (long)s * a.k_raw_stride_t + (long)hh * (D * 2);
+        dst = kvrow + (long)hh * (2 * D * 2);
+      } else {
+        kind = 2;
+        const int hh = u - a.Hq - a.Hkv;
+        src = a.v_raw + (long)s * a.v_raw_stride_t + (long)hh * (D * 2);
+        dst = kvrow + (long)hh * (2 * D * 2) + D * 2;
+      }
+      const u32x4 va = *(const u32x4*)(src + ea * 2);
+      const u32x4 vb = *(const u32x4*)(src + eb * 2);
+      if (kind == 2) {
+        *(u32x4*)(dst + ea * 2) = va;
+        *(u32x4*)(dst + eb * 2) = vb;
+        continue;
+      }
+      float x[16];
+      unpack8(va, x);
+      unpack8(vb, x + 8);
+      norm16(x, s_par[2 * kind], s_par[2 * kind + 1], ea, eb, a.norm_kind, a.eps, true);
+      if (rot_lane && a.rope) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float x1 = x[i], x2 = x[8 + i];
+          x[i] = x1 * cs[i] - x2 * sn[i];
+          x[8 + i] = x1 * sn[i] + x2 * cs[i];
+        }
+      }
+      *(u32x4*)(dst + ea * 2) = pack8(x);
+      *(u32x4*)(dst + eb * 2) = pack8(x + 8);
+    }
+  }
+}
+
+// x [S, H, 128] bf16 with strides -> y contiguous, norm only.
+__global__ __launch_bounds__(THREADS) void head_norm_kernel(const char* x, long xs_t, long xs_h, const float* gamma,
+                                                            const float* beta, char* y, int S, int H, int norm_kind,
+                                                            float eps) {
+  __shared__ float s_par[2][D];
+  const int tid = threadIdx.x;
+  for (int i = tid; i < 2 * D; i += THREADS) {
+    const float* src = i < D ? gamma : beta;
+    s_par[i / D][i % D] = src ? src[i % D] : 0.f;
+  }
+  __syncthreads();
+  const int j = tid & 7;
+  const long row = (long)blockIdx.x * GROUPS + (tid >> 3);
+  if (row >= (long)S * H) return;
+  const long s = row / H, h = row % H;
+  const char* src = x + s * xs_t + h * xs_h;
+  char* dst = y + row * (D * 2);
+  const int ea = 16 * j, eb = ea + 8;
+  float v[16];
+  unpack8(*(const u32x4*)(src + ea * 2), v);
+  unpack8(*(const u32x4*)(src + eb * 2), v + 8);
+  norm16(v, s_par[0], s_par[1], ea, eb, norm_kind, eps, beta != nullptr);
+  *(u32x4*)(dst + ea * 2) = pack8(v);
+  *(u32x4*)(dst + eb * 2) = pack8(v + 8);
+}
+
+// Rotary only: x, y [B, S, H, D]; one thread per (row, pair).
+template <bool BF16>
+__global__ __launch_bounds__(THREADS) void rotary_kernel(const void* xin, const float* cosp, const float* sinp,
+                                                         void* yout, long rows, int S, int H, int Dd, int R2) {
+  const long gid = (long)blockIdx.x * THREADS + threadIdx.x;
+  const int half = Dd / 2;  // threads per row: each handles elements p and p + half ... see below
+  const long row = gid / half;
+  const int p = (int)(gid % half);
+  if (row >= rows) return;
+  const long s = (row / H) % S;
+  // thread p < R2 rotates the pair (p, p + R2); threads R2 <= p < half copy the tail two at a time
+  auto ld = [&](long idx) -> float {
+    if (BF16) return __builtin_bit_cast(float, (unsigned)((const unsigned short*)xin)[idx] << 16);
+    return ((const float*)xin)[idx];
+  };
+  auto st = [&](long idx, float v) {
+    if (BF16) {
+      f32x2 t = {v, 0.f};
+      bf16x2 r = __builtin_convertvector(t, bf16x2);
+      ((unsigned short*)yout)[idx] = (unsigned short)(__builtin_bit_cast(unsigned, r) & 0xffffu);
+    } else {
+      ((float*)yout)[idx] = v;
+    }
+  };
+  const long base = row * Dd;
+  if (p < R2) {
+    const float c = cosp[s * R2 + p], sn = sinp[s * R2 + p];
+    const float x1 = ld(base + p), x2 = ld(base + R2 + p);
+    st(base + p, x1 * c - x2 * sn);
+    st(base + R2 + p, x1 * sn + x2 * c);
+  } else {
+    const int e = 2 * R2 + 2 * (p - R2);
+    st(base + e, ld(base + e));
+    st(base + e + 1, ld(base + e + 1));
+  }
+}
+
+}  // namespace
+
+hipError_t launch_prologue(const PrologueKernArgs& a, hipStream_t stream) {
+  if (a.S <= 0) return hipSuccess;
+  const unsigned grid = (unsigned)((a.S + TOK_PER_BLOCK - 1) / TOK_PER_BLOCK);
+  hipLaunchKernelGGL(prologue_kernel, dim3(grid), dim3(THREADS), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_head_norm(const char* x, long x_stride_t, long x_stride_h, const float* gamma, const float* beta,
+                            char* y, int S, int H, int norm_kind, float eps, hipStream_t stream) {
+  const long rows = (long)S * H;
+  if (rows <= 0) return hipSuccess;
+  const unsigned grid = (unsigned)((rows + GROUPS - 1) / GROUPS);
+  hipLaunchKernelGGL(head_norm_kernel, dim3(grid), dim3(THREADS), 0, stream, x, x_stride_t, x_stride_h, gamma, beta, y,
+                     S, H, norm_kind, eps);
+  return hipGetLastError();
+}
+
+hipError_t launch_rotary(const void* x, const float* cos, const float* sin, void* y, int B, int S, int H, int Dd, int R2,
+                         int is_bf16, hipStream_t stream) {
+  const long rows = (long)B * S * H;
+  const long threads = rows * (Dd / 2);
+  if (threads <= 0) return hipSuccess;
+  const unsigned grid = (unsigned)((threads + THREADS - 1) / THREADS);
+  if (is_bf16)
+    hipLaunchKernelGGL(rotary_kernel<true>, dim3(grid), dim3(THREADS), 0, stream, x, cos, sin, y, rows, S, H, Dd, R2);
+  else
+    hipLaunchKernelGGL(rotary_kernel<false>, dim3(grid), dim3(THREADS), 0, stream, x, cos, sin, y, rows, S, H, Dd, R2);
+  return hipGetLastError();
+}
+
+}  // namespace magi

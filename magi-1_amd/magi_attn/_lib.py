@@ -1,0 +1,96 @@
+"""ctypes binding of libmagi_attn.so (the C-ABI declared in include/magi_attn.h).
+
+The library is the only compute path: when it is missing, loading raises, there is no
+fallback to PyTorch ops.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmagi_attn.so")
+
+MAGI_DTYPE_BF16 = 0
+MAGI_DTYPE_FP8_E4M3 = 1
+MAGI_RANGES_PAIRS = 0
+MAGI_RANGES_CU = 1
+MAGI_NORM_LAYERNORM_1P = 0
+MAGI_NORM_RMSNORM_1P = 1
+MAGI_NORM_NONE = 2
+
+
+class MagiError(RuntimeError):
+    """A C-ABI call returned a negative code; .code holds it."""
+
+    def __init__(self, code: int, msg: str):
+        super().__init__(f"libmagi_attn error {code}: {msg}")
+        self.code = code
+
+
+class AttnArgs(C.Structure):
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("k2", C.c_void_p), ("v2", C.c_void_p),
+        ("out", C.c_void_p), ("lse", C.c_void_p), ("q_ranges", C.c_void_p), ("k_ranges", C.c_void_p),
+        ("q_scale", C.c_void_p), ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
+        ("q_stride_t", C.c_int64), ("q_stride_h", C.c_int64), ("k_stride_t", C.c_int64), ("k_stride_h", C.c_int64),
+        ("v_stride_t", C.c_int64), ("v_stride_h", C.c_int64), ("o_stride_t", C.c_int64), ("o_stride_h", C.c_int64),
+        ("total_q", C.c_int32), ("total_k", C.c_int32), ("k_split", C.c_int32),
+        ("n_ranges", C.c_int32), ("ranges_mode", C.c_int32),
+        ("max_seqlen_q", C.c_int32), ("max_seqlen_k", C.c_int32),
+        ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32),
+        ("dtype", C.c_int32), ("scale_chunk_tokens", C.c_int32),
+        ("softmax_scale", C.c_float), ("reserved", C.c_int32),
+    ]
+
+
+class PrologueArgs(C.Structure):
+    _fields_ = [
+        ("q_raw", C.c_void_p), ("k_raw", C.c_void_p), ("v_raw", C.c_void_p), ("rope", C.c_void_p),
+        ("gq", C.c_void_p), ("bq", C.c_void_p), ("gk", C.c_void_p), ("bk", C.c_void_p),
+        ("q_out", C.c_void_p), ("kv_out", C.c_void_p), ("kv_tail", C.c_void_p),
+        ("q_raw_stride_t", C.c_int64), ("k_raw_stride_t", C.c_int64), ("v_raw_stride_t", C.c_int64),
+        ("kv_stride_t", C.c_int64), ("kv_tail_stride_t", C.c_int64),
+        ("S", C.c_int32), ("n_cache_rows", C.c_int32),
+        ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32), ("R2", C.c_int32),
+        ("norm_kind", C.c_int32), ("eps", C.c_float),
+    ]
+
+
+EXPORTS = ("magi_version", "magi_last_error", "magi_attn_fwd", "magi_qk_prologue", "magi_head_norm",
+           "magi_apply_rotary", "magi_quantize_fp8")
+
+_lib = None
+
+
+def lib() -> C.CDLL:
+    """Load (once) and return the shared library; raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `make -C magi-1_amd/csrc` (or __graft_entry__.build()); "
+                "there is no fallback path")
+        l = C.CDLL(LIB_PATH)
+        l.magi_version.restype = C.c_int
+        l.magi_last_error.restype = C.c_char_p
+        l.magi_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+        l.magi_attn_fwd.restype = C.c_int
+        l.magi_qk_prologue.argtypes = [C.POINTER(PrologueArgs), C.c_void_p]
+        l.magi_qk_prologue.restype = C.c_int
+        l.magi_head_norm.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,
+                                     C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_void_p]
+        l.magi_head_norm.restype = C.c_int
+        l.magi_apply_rotary.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
+                                        C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+        l.magi_apply_rotary.restype = C.c_int
+        l.magi_quantize_fp8.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32,
+                                        C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+        l.magi_quantize_fp8.restype = C.c_int
+        _lib = l
+    return _lib
+
+
+def check(code: int) -> None:
+    if code != 0:
+        raise MagiError(code, lib().magi_last_error().decode("utf-8", "replace"))

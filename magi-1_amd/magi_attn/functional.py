@@ -1,0 +1,254 @@
+"""Reference-shaped callables over the C-ABI.
+
+The four functions the reference's DiT module imports from third-party CUDA packages
+(inference/model/dit/dit_module.py:27-37) keep their names, argument meaning and return
+shapes here, so the module-level code reads the same:
+
+  flex_flash_attn_func   (MagiAttention; dit_module.py:1032-1043, 1111-1122)
+  flash_attn_func        (flash-attn;    dit_module.py:1062, 1090-1095)
+  flash_attn_varlen_func (flash-attn;    dit_module.py:1124-1133)
+  apply_rotary_emb       (flash-attn;    dit_module.py:961, 978)
+
+plus the fused prologue and the cache-aware range attention this library adds.  PyTorch is
+used for device memory and the current stream only.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib as L
+
+
+def _stream() -> C.c_void_p:
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _check_thd(t: torch.Tensor, name: str) -> None:
+    if t.dim() != 3:
+        raise ValueError(f"{name} must be [tokens, heads, head_dim], got {tuple(t.shape)}")
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a CUDA (ROCm) tensor")
+    if t.stride(2) != 1:
+        raise ValueError(f"{name}: head_dim must be contiguous")
+
+
+def _dtype_code(t: torch.Tensor) -> int:
+    if t.dtype == torch.bfloat16:
+        return L.MAGI_DTYPE_BF16
+    if t.dtype == torch.float8_e4m3fn:
+        return L.MAGI_DTYPE_FP8_E4M3
+    raise TypeError(f"unsupported dtype {t.dtype}: bf16 or float8_e4m3fn")
+
+
+def range_attention(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    q_ranges: torch.Tensor,
+    k_ranges: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int = 0,
+    softmax_scale: Optional[float] = None,
+    *,
+    ranges_mode: int = L.MAGI_RANGES_PAIRS,
+    k2: Optional[torch.Tensor] = None,
+    v2: Optional[torch.Tensor] = None,
+    k_split: Optional[int] = None,
+    q_scale: Optional[torch.Tensor] = None,
+    k_scale: Optional[torch.Tensor] = None,
+    v_scale: Optional[torch.Tensor] = None,
+    scale_chunk_tokens: int = 0,
+    out: Optional[torch.Tensor] = None,
+    return_lse: bool = True,
+    zero_init: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """out[q_range_i] = softmax(q k^T * scale) v over k[k_range_i]; see magi_attn_fwd.
+
+    k and v may be strided views (e.g. the two halves of an interleaved KV cache); with
+    k2 / v2 the key axis is the concatenation [k[:k_split] | k2] without copying.
+    """
+    _check_thd(q, "q")
+    _check_thd(k, "k")
+    _check_thd(v, "v")
+    Tq, Hq, D = q.shape
+    Hkv = k.shape[1]
+    if k.stride() != v.stride() and (k.stride(0) != v.stride(0) or k.stride(1) != v.stride(1)):
+        pass  # independent strides are supported
+    total_k = k.shape[0] if k2 is None else int(k_split) + k2.shape[0]
+    if k2 is not None:
+        _check_thd(k2, "k2")
+        _check_thd(v2, "v2")
+        if k2.stride() != k.stride() or v2.stride() != v.stride():
+            raise ValueError("k2 / v2 must have the strides of k / v")
+        if k_split is None or not (0 <= k_split <= k.shape[0]):
+            raise ValueError("k_split must lie inside k")
+    if q_ranges.dtype != torch.int32 or k_ranges.dtype != torch.int32:
+        raise TypeError("q_ranges / k_ranges must be int32")
+    if not (q_ranges.is_cuda and k_ranges.is_cuda):
+        raise ValueError("q_ranges / k_ranges must live on the device")
+    q_ranges = q_ranges.contiguous()
+    k_ranges = k_ranges.contiguous()
+    if ranges_mode == L.MAGI_RANGES_PAIRS:
+        n = q_ranges.shape[0]
+        if q_ranges.shape != k_ranges.shape or q_ranges.dim() != 2 or q_ranges.shape[1] != 2:
+            raise ValueError("q_ranges / k_ranges must both be [n, 2]")
+    else:
+        n = q_ranges.numel() - 1
+        if q_ranges.numel() != k_ranges.numel():
+            raise ValueError("cu_seqlens_q / cu_seqlens_k must have the same length")
+    if out is None:
+        out = (torch.zeros if zero_init else torch.empty)((Tq, Hq, D), dtype=torch.bfloat16, device=q.device)
+    lse = None
+    if return_lse:
+        lse = torch.full((Hq, Tq), float("-inf"), dtype=torch.float32, device=q.device)
+    a = L.AttnArgs()
+    a.q, a.k, a.v, a.k2, a.v2 = _ptr(q), _ptr(k), _ptr(v), _ptr(k2), _ptr(v2)
+    a.out, a.lse = _ptr(out), _ptr(lse)
+    a.q_ranges, a.k_ranges = _ptr(q_ranges), _ptr(k_ranges)
+    a.q_scale, a.k_scale, a.v_scale = _ptr(q_scale), _ptr(k_scale), _ptr(v_scale)
+    a.q_stride_t, a.q_stride_h = q.stride(0), q.stride(1)
+    a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1)
+    a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1)
+    a.o_stride_t, a.o_stride_h = out.stride(0), out.stride(1)
+    a.total_q, a.total_k = Tq, total_k
+    a.k_split = total_k if k2 is None else int(k_split)
+    a.n_ranges, a.ranges_mode = max(n, 0), ranges_mode
+    a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+    a.Hq, a.Hkv, a.D = Hq, Hkv, D
+    a.dtype = _dtype_code(q)
+    a.scale_chunk_tokens = int(scale_chunk_tokens)
+    a.softmax_scale = 0.0 if softmax_scale is None else float(softmax_scale)
+    with torch.cuda.device(q.device):
+        L.check(L.lib().magi_attn_fwd(C.byref(a), _stream()))
+    return out, lse
+
+
+def flex_flash_attn_func(q, k, v, q_ranges, k_ranges, max_seqlen_q, max_seqlen_k, softmax_scale=None,
+                         deterministic=False, disable_fwd_atomic_reduction=True, **_unused):
+    """(out [Tq,Hq,D], lse [Hq,Tq]) for disjoint q ranges.  The forward has one writer per output
+    row, so it is deterministic and needs no atomic reduction whatever the two flags say."""
+    return range_attention(q, k, v, q_ranges, k_ranges, max_seqlen_q, max_seqlen_k, softmax_scale)
+
+
+def flash_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, deterministic=False, **_unused):
+    """q [B,Sq,Hq,D], k/v [B,Sk,Hkv,D] -> [B,Sq,Hq,D]; non-causal, no dropout (what the reference uses)."""
+    if dropout_p != 0.0 or causal:
+        raise NotImplementedError("dropout / causal are not part of the MAGI-1 attention path")
+    B, Sq, Hq, D = q.shape
+    Sk = k.shape[1]
+    q3 = q.reshape(B * Sq, Hq, D)
+    k3 = k.reshape(B * Sk, k.shape[2], D)
+    v3 = v.reshape(B * Sk, v.shape[2], D)
+    cu_q = torch.arange(0, (B + 1) * Sq, Sq, dtype=torch.int32, device=q.device)
+    cu_k = torch.arange(0, (B + 1) * Sk, Sk, dtype=torch.int32, device=q.device)
+    out, _ = range_attention(q3, k3, v3, cu_q, cu_k, Sq, Sk, softmax_scale, ranges_mode=L.MAGI_RANGES_CU,
+                             return_lse=False, zero_init=False)
+    return out.view(B, Sq, Hq, D)
+
+
+def flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p=0.0,
+                           softmax_scale=None, causal=False, deterministic=False, **_unused):
+    """Packed varlen attention; segment s pairs q[cu_q[s]:cu_q[s+1]] with k[cu_k[s]:cu_k[s+1]].
+    A segment without keys yields zero rows."""
+    if dropout_p != 0.0 or causal:
+        raise NotImplementedError("dropout / causal are not part of the MAGI-1 attention path")
+    out, _ = range_attention(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale,
+                             ranges_mode=L.MAGI_RANGES_CU, return_lse=False, zero_init=True)
+    return out
+
+
+def apply_rotary_emb(x, cos, sin, interleaved=False, inplace=False, **_unused):
+    """x [B,S,H,D] (fp32 or bf16), cos / sin [S, R/2]: rotate the first R features, non-interleaved."""
+    if interleaved:
+        raise NotImplementedError("the DiT path uses the non-interleaved convention only")
+    if x.dim() != 4:
+        raise ValueError("x must be [batch, seqlen, heads, head_dim]")
+    if x.dtype not in (torch.float32, torch.bfloat16):
+        raise TypeError("x must be fp32 or bf16")
+    B, S, H, D = x.shape
+    R2 = cos.shape[-1]
+    if cos.shape != (S, R2) or sin.shape != (S, R2):
+        raise ValueError("cos / sin must be [seqlen, rotary_dim / 2]")
+    xc = x.contiguous()
+    y = xc if inplace else torch.empty_like(xc)
+    cosf = cos.to(torch.float32).contiguous()
+    sinf = sin.to(torch.float32).contiguous()
+    with torch.cuda.device(x.device):
+        L.check(L.lib().magi_apply_rotary(xc.data_ptr(), cosf.data_ptr(), sinf.data_ptr(), y.data_ptr(), B, S, H, D, R2,
+                                          int(x.dtype == torch.bfloat16), _stream()))
+    return y
+
+
+def qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int, eps: float = 1e-6,
+                norm_kind: int = L.MAGI_NORM_LAYERNORM_1P, kv_out: Optional[torch.Tensor] = None,
+                n_cache_rows: Optional[int] = None, kv_tail: Optional[torch.Tensor] = None,
+                q_out: Optional[torch.Tensor] = None):
+    """Fused norm + rotary + cast + KV write.  q_raw [S, Hq*D], k_raw / v_raw [S, Hkv*D] bf16 (row
+    strided views allowed); rope [S, 2*R2] fp32 (sin | cos) or None.
+
+    kv_out is the destination of the first n_cache_rows tokens (a view of the cache starting
+    at the write position, [>= n_cache_rows, Hkv, 2D]); kv_tail takes the rest.  With neither,
+    a fresh [S, Hkv, 2D] tensor is written.  Returns (q [S,Hq,D], kv_out, kv_tail)."""
+    S = q_raw.shape[0]
+    D = 128
+    dev = q_raw.device
+    if q_out is None:
+        q_out = torch.empty((S, Hq, D), dtype=torch.bfloat16, device=dev)
+    if kv_out is None and kv_tail is None:
+        kv_out = torch.empty((S, Hkv, 2 * D), dtype=torch.bfloat16, device=dev)
+        n_cache_rows = S
+    if n_cache_rows is None:
+        n_cache_rows = S if kv_tail is None else 0
+    for name, t in (("q_raw", q_raw), ("k_raw", k_raw), ("v_raw", v_raw)):
+        if t.dtype != torch.bfloat16 or t.stride(-1) != 1 or t.dim() != 2:
+            raise ValueError(f"{name} must be a 2-D bf16 tensor with contiguous rows")
+    for name, t in (("kv_out", kv_out), ("kv_tail", kv_tail)):
+        if t is not None and (t.dtype != torch.bfloat16 or t.dim() != 3 or t.shape[1:] != (Hkv, 2 * D)
+                              or t.stride(2) != 1 or t.stride(1) != 2 * D):
+            raise ValueError(f"{name} must be bf16 [rows, Hkv, 2*D] with contiguous heads")
+    if kv_out is not None and kv_out.shape[0] < n_cache_rows:
+        raise ValueError("kv_out is shorter than n_cache_rows")
+    if kv_tail is not None and kv_tail.shape[0] < S - n_cache_rows:
+        raise ValueError("kv_tail is shorter than S - n_cache_rows")
+    f32 = lambda t: None if t is None else t.to(torch.float32).contiguous()
+    gq, bq, gk, bk = f32(gq), f32(bq), f32(gk), f32(bk)
+    a = L.PrologueArgs()
+    R2 = 0
+    if rope is not None:
+        if rope.dtype != torch.float32 or rope.dim() != 2 or rope.shape[0] != S or not rope.is_contiguous():
+            raise ValueError("rope must be a contiguous fp32 [S, 2*R2] tensor")
+        R2 = rope.shape[1] // 2
+    a.q_raw, a.k_raw, a.v_raw, a.rope = _ptr(q_raw), _ptr(k_raw), _ptr(v_raw), _ptr(rope)
+    a.gq, a.bq, a.gk, a.bk = _ptr(gq), _ptr(bq), _ptr(gk), _ptr(bk)
+    a.q_out, a.kv_out, a.kv_tail = _ptr(q_out), _ptr(kv_out), _ptr(kv_tail)
+    a.q_raw_stride_t, a.k_raw_stride_t, a.v_raw_stride_t = q_raw.stride(0), k_raw.stride(0), v_raw.stride(0)
+    a.kv_stride_t = 0 if kv_out is None else kv_out.stride(0)
+    a.kv_tail_stride_t = 0 if kv_tail is None else kv_tail.stride(0)
+    a.S, a.n_cache_rows = S, int(n_cache_rows)
+    a.Hq, a.Hkv, a.D, a.R2 = Hq, Hkv, D, R2
+    a.norm_kind, a.eps = int(norm_kind), float(eps)
+    with torch.cuda.device(dev):
+        L.check(L.lib().magi_qk_prologue(C.byref(a), _stream()))
+    return q_out, kv_out, kv_tail
+
+
+def head_norm(x: torch.Tensor, gamma, beta, eps: float = 1e-6, norm_kind: int = L.MAGI_NORM_LAYERNORM_1P):
+    """x [S, H, 128] bf16 (strided heads allowed) -> contiguous normalised copy."""
+    _check_thd(x, "x")
+    if x.dtype != torch.bfloat16:
+        raise TypeError("x must be bf16")
+    S, H, D = x.shape
+    y = torch.empty((S, H, D), dtype=torch.bfloat16, device=x.device)
+    g = None if gamma is None else gamma.to(torch.float32).contiguous()
+    b = None if beta is None else beta.to(torch.float32).contiguous()
+    with torch.cuda.device(x.device):
+        L.check(L.lib().magi_head_norm(x.data_ptr(), x.stride(0), x.stride(1), _ptr(g), _ptr(b), y.data_ptr(), S, H, D,
+                                       int(norm_kind), float(eps), _stream()))
+    return y

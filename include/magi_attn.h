@@ -112,7 +112,7 @@ int magi_attn_fwd(const magi_attn_args* args, void* stream);
  * cache append of _full_adjust_key_and_value (dit_module.py:918-929).
  *
  * q_raw [S, Hq*D], k_raw / v_raw [S, Hkv*D]  bf16, token strides in elements
- * rope  [S, 2*R2] fp32, sin in the first R2 columns, cos in the last R2 (dit_module.py:770, 1147);
+ * rope  [S / batch, 2*R2] fp32, sin in the first R2 columns, cos in the last R2 (dit_module.py:770, 1147);
  *       rotary_dim = 2*R2 <= D; NULL disables rotary
  * gq,bq,gk,bk  fp32 [D] norm parameters (gamma stored zero-centred); b* may be NULL
  * q_out [S, Hq, D] bf16 contiguous (or fp8 with q_scale_out, see below)
@@ -139,6 +139,8 @@ typedef struct magi_prologue_args {
   int32_t Hq, Hkv, D, R2;
   int32_t norm_kind;
   float eps;
+  int32_t batch; /* tokens are ordered (position, batch): rope row of token t is t / batch; 0 or 1 = no batch */
+  int32_t reserved;
 } magi_prologue_args;
 
 int magi_qk_prologue(const magi_prologue_args* args, void* stream);

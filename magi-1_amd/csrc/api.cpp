@@ -47,7 +47,9 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     return fail(MAGI_EINVAL, "magi_attn_fwd: unknown ranges_mode %d", p->ranges_mode);
   if (p->n_ranges == 0 || p->total_q == 0 || p->max_seqlen_q == 0) return MAGI_OK;
   if (!p->q || !p->out || !p->q_ranges || !p->k_ranges) return fail(MAGI_EINVAL, "magi_attn_fwd: NULL q/out/ranges");
-  if (p->total_k > 0 && (!p->k || !p->v)) return fail(MAGI_EINVAL, "magi_attn_fwd: NULL k/v with total_k > 0");
+  const bool all_in_second = p->k2 && p->v2 && p->k_split == 0;  // an empty first segment may be NULL
+  if (p->total_k > 0 && (!p->k || !p->v) && !all_in_second)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: NULL k/v with total_k > 0");
   const int esz = p->dtype == MAGI_DTYPE_BF16 ? 2 : 1;
   const int64_t row_elems = 16 / esz;  // 16-byte vectors
   if (p->q_stride_h % row_elems || p->q_stride_t % row_elems || p->k_stride_h % row_elems ||
@@ -124,6 +126,7 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   if (p->R2 < 0 || p->R2 % 8 || 2 * p->R2 > p->D)
     return fail(MAGI_EINVAL, "magi_qk_prologue: R2=%d must be a multiple of 8 with 2*R2 <= D", p->R2);
   if (p->norm_kind < 0 || p->norm_kind > 2) return fail(MAGI_EINVAL, "magi_qk_prologue: norm_kind %d", p->norm_kind);
+  if (p->batch < 0) return fail(MAGI_EINVAL, "magi_qk_prologue: negative batch");
   if (p->Hq > 0 && (!p->q_raw || !p->q_out)) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL q_raw/q_out");
   if (p->Hkv > 0 && (!p->k_raw || !p->v_raw)) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL k_raw/v_raw");
   if (p->n_cache_rows < 0 || p->n_cache_rows > p->S)
@@ -167,6 +170,7 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   a.R2 = a.rope ? p->R2 : 0;
   a.norm_kind = p->norm_kind;
   a.eps = p->eps;
+  a.batch = p->batch > 1 ? p->batch : 1;
   hipError_t e = magi::launch_prologue(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_qk_prologue launch");
   return MAGI_OK;

@@ -131,21 +131,22 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const At
   const int st_v = r0 * ROW_BYTES + ((cc ^ ((r0 & 3) << 2)) << 4);  // V tile: chunk ^= (row & 3) << 2
   u32x4 kr[4], vr[4];
 
+  // rows >= k_split come from the second segment: same strides, so only the base differs
+  const char* const kbase = a.k;
+  const char* const vbase = a.v;
+  const long k2_delta = a.k2 ? (a.k2 - a.k) - (long)a.k_split * a.ks_t : 0;
+  const long v2_delta = a.v2 ? (a.v2 - a.v) - (long)a.k_split * a.vs_t : 0;
+  const int k_split = a.k_split;
+  const long ks_t = a.ks_t, vs_t = a.vs_t;
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int row = min(k0 + r0 + 16 * j, ke - 1);
-      const char* kb;
-      const char* vb;
-      if (row < a.k_split) {
-        kb = a.k + (long)row * a.ks_t;
-        vb = a.v + (long)row * a.vs_t;
-      } else {
-        kb = a.k2 + (long)(row - a.k_split) * a.ks_t;
-        vb = a.v2 + (long)(row - a.k_split) * a.vs_t;
-      }
-      kr[j] = *(const u32x4*)(kb + kcol);
-      vr[j] = *(const u32x4*)(vb + vcol);
+      const bool second = row >= k_split;
+      const long ko = (long)row * ks_t + kcol + (second ? k2_delta : 0);
+      const long vo = (long)row * vs_t + vcol + (second ? v2_delta : 0);
+      kr[j] = *(const u32x4*)(kbase + ko);
+      vr[j] = *(const u32x4*)(vbase + vo);
     }
   };
   auto stash = [&](int buf) {
@@ -234,10 +235,12 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const At
       pb[s] = __builtin_bit_cast(bf16x8, pk);
     }
     l_run = l_run * alpha + psum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // some row of this wave saw a new maximum
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+        for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+    }
 
     // O^T[d][q] += V^T[d][key] P^T[key][q]
 #pragma unroll

@@ -53,6 +53,7 @@ struct PrologueKernArgs {
   int Hq, Hkv, R2;
   int norm_kind;
   float eps;
+  int batch;
 };
 hipError_t launch_prologue(const PrologueKernArgs& a, hipStream_t stream);
 

@@ -94,7 +94,7 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
     if (s >= a.S) break;
     float sn[8], cs[8];
     if (rot_lane && a.rope) {
-      const float* rp = a.rope + (long)s * (2 * a.R2);
+      const float* rp = a.rope + (long)(s / a.batch) * (2 * a.R2);
       const f32x4 s0 = *(const f32x4*)(rp + 8 * j), s1 = *(const f32x4*)(rp + 8 * j + 4);
       const f32x4 c0 = *(const f32x4*)(rp + a.R2 + 8 * j), c1 = *(const f32x4*)(rp + a.R2 + 8 * j + 4);
 #pragma unroll

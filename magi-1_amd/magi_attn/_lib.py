@@ -53,7 +53,7 @@ class PrologueArgs(C.Structure):
         ("kv_stride_t", C.c_int64), ("kv_tail_stride_t", C.c_int64),
         ("S", C.c_int32), ("n_cache_rows", C.c_int32),
         ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32), ("R2", C.c_int32),
-        ("norm_kind", C.c_int32), ("eps", C.c_float),
+        ("norm_kind", C.c_int32), ("eps", C.c_float), ("batch", C.c_int32), ("reserved", C.c_int32),
     ]
 
 

@@ -189,7 +189,7 @@ def apply_rotary_emb(x, cos, sin, interleaved=False, inplace=False, **_unused):
 def qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int, eps: float = 1e-6,
                 norm_kind: int = L.MAGI_NORM_LAYERNORM_1P, kv_out: Optional[torch.Tensor] = None,
                 n_cache_rows: Optional[int] = None, kv_tail: Optional[torch.Tensor] = None,
-                q_out: Optional[torch.Tensor] = None):
+                q_out: Optional[torch.Tensor] = None, batch: int = 1):
     """Fused norm + rotary + cast + KV write.  q_raw [S, Hq*D], k_raw / v_raw [S, Hkv*D] bf16 (row
     strided views allowed); rope [S, 2*R2] fp32 (sin | cos) or None.
 
@@ -222,8 +222,8 @@ def qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int,
     a = L.PrologueArgs()
     R2 = 0
     if rope is not None:
-        if rope.dtype != torch.float32 or rope.dim() != 2 or rope.shape[0] != S or not rope.is_contiguous():
-            raise ValueError("rope must be a contiguous fp32 [S, 2*R2] tensor")
+        if rope.dtype != torch.float32 or rope.dim() != 2 or rope.shape[0] * max(batch, 1) != S or not rope.is_contiguous():
+            raise ValueError("rope must be a contiguous fp32 [S / batch, 2*R2] tensor")
         R2 = rope.shape[1] // 2
     a.q_raw, a.k_raw, a.v_raw, a.rope = _ptr(q_raw), _ptr(k_raw), _ptr(v_raw), _ptr(rope)
     a.gq, a.bq, a.gk, a.bk = _ptr(gq), _ptr(bq), _ptr(gk), _ptr(bk)
@@ -233,7 +233,7 @@ def qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int,
     a.kv_tail_stride_t = 0 if kv_tail is None else kv_tail.stride(0)
     a.S, a.n_cache_rows = S, int(n_cache_rows)
     a.Hq, a.Hkv, a.D, a.R2 = Hq, Hkv, D, R2
-    a.norm_kind, a.eps = int(norm_kind), float(eps)
+    a.norm_kind, a.eps, a.batch = int(norm_kind), float(eps), int(batch)
     with torch.cuda.device(dev):
         L.check(L.lib().magi_qk_prologue(C.byref(a), _stream()))
     return q_out, kv_out, kv_tail

@@ -1,0 +1,300 @@
+"""The DiT attention layer over libmagi_attn, with the interface of the reference's
+FullyParallelAttention for cp_strategy == "none"
+(inference/model/dit/dit_module.py:776-1173).
+
+Method names, argument meaning and returned layouts follow the reference so that
+TransformerLayer-level code can call it unchanged:
+
+  forward(hidden_states [S,b,h], key_value_states [Ty,h*ratio], inference_params,
+          rotary_pos_emb [S,96], meta_args) -> (core_attn_out [S,b,Hq*D], xattn_out [S,b,Hq*D])
+
+What differs is what happens underneath:
+  * get_q / get_k / get_v / get_kv: the upcast, LayerNorm, transpose, rotary, downcast and
+    re-layout passes are one fused kernel launch;
+  * the KV cache is appended to in place by that same launch and READ in place by the
+    attention kernel (strided K / V views of the interleaved cache), so the prefix slice,
+    the cat and the contiguous copies of _full_adjust_key_and_value / core_attention vanish;
+  * when the cache must not be updated (update_kv_cache False, or the last chunk under
+    distill_nearly_clean_chunk) the new KV goes to a side buffer and the kernel walks
+    [cache prefix | side buffer] as one key axis.
+
+The linear projections and the input LayerNorm are plain library GEMMs / ops (torch on
+rocBLAS / hipBLASLt); they are not part of this library.
+"""
+from __future__ import annotations
+
+from typing import Callable, Optional, Tuple
+
+import torch
+
+from . import _lib as L
+from .functional import head_norm, qk_prologue, range_attention
+from .params import InferenceParams, ModelMetaArgs, PackedCrossAttnParams
+
+
+class FusedLayerNorm(torch.nn.Module):
+    """Parameter holder of a per-head LayerNorm with zero-centred gamma (dit_module.py:323-357).
+    The arithmetic runs inside the fused kernels; forward() is the stand-alone form."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-6, zero_centered_gamma: bool = True,
+                 dtype=torch.bfloat16, device=None):
+        super().__init__()
+        self.eps = eps
+        self.zero_centered_gamma = zero_centered_gamma
+        self.weight = torch.nn.Parameter(torch.zeros(hidden_size, dtype=dtype, device=device))
+        self.bias = torch.nn.Parameter(torch.zeros(hidden_size, dtype=dtype, device=device))
+
+    def gamma_beta_fp32(self) -> Tuple[torch.Tensor, torch.Tensor]:
+        """(gamma - 1 form, beta) as the kernels take them.  weight + 1 is formed in the parameter
+        dtype first, as the reference does, so a bf16 parameter rounds the same way."""
+        w = self.weight.detach()
+        g = ((w + 1).float() - 1.0) if self.zero_centered_gamma else (w.float() - 1.0)
+        return g, self.bias.detach().float()
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        g, b = self.gamma_beta_fp32()
+        shape = x.shape
+        y = head_norm(x.reshape(-1, shape[-2], shape[-1]).to(torch.bfloat16), g, b, self.eps)
+        return y.reshape(shape).to(x.dtype)
+
+
+class CustomLayerNormLinear(torch.nn.Module):
+    """Input LayerNorm + the four projections q, qx, k, v (dit_module.py:390-425)."""
+
+    def __init__(self, input_size: int, output_size_q: int, output_size_kv: int, eps: float = 1e-6,
+                 dtype=torch.bfloat16, device=None):
+        super().__init__()
+        self.layer_norm = torch.nn.LayerNorm(input_size, eps=eps, dtype=dtype, device=device)
+        self.q = torch.nn.Linear(input_size, output_size_q, bias=False, dtype=dtype, device=device)
+        self.qx = torch.nn.Linear(input_size, output_size_q, bias=False, dtype=dtype, device=device)
+        self.k = torch.nn.Linear(input_size, output_size_kv, bias=False, dtype=dtype, device=device)
+        self.v = torch.nn.Linear(input_size, output_size_kv, bias=False, dtype=dtype, device=device)
+
+    def forward_ln(self, hidden_states):
+        return self.layer_norm(hidden_states)
+
+    def forward_q(self, hidden_states):
+        return self.q(hidden_states)
+
+    def forward_qx(self, hidden_states):
+        return self.qx(hidden_states)
+
+    def forward_k(self, hidden_states):
+        return self.k(hidden_states)
+
+    def forward_v(self, hidden_states):
+        return self.v(hidden_states)
+
+
+class FullyParallelAttention(torch.nn.Module):
+    def __init__(self, hidden_size: int, num_attention_heads: int, num_query_groups: int, kv_channels: int = 128,
+                 layer_number: int = 0, layernorm_epsilon: float = 1e-6, apply_layernorm_1p: bool = True,
+                 xattn_cond_hidden_ratio: float = 1.0, params_dtype=torch.bfloat16, device=None):
+        super().__init__()
+        if kv_channels != 128:
+            raise NotImplementedError("head_dim 128 only")
+        self.layer_number = layer_number
+        self.hidden_size_per_attention_head = kv_channels
+        self.num_attention_heads = num_attention_heads
+        self.num_query_groups_per_partition = num_query_groups
+        self.query_projection_size = kv_channels * num_attention_heads
+        self.kv_projection_size = kv_channels * num_query_groups
+        self.eps = layernorm_epsilon
+        self.linear_qkv = CustomLayerNormLinear(hidden_size, self.query_projection_size, self.kv_projection_size,
+                                                eps=layernorm_epsilon, dtype=params_dtype, device=device)
+        self.linear_kv_xattn = torch.nn.Linear(int(hidden_size * xattn_cond_hidden_ratio), 2 * self.kv_projection_size,
+                                               bias=False, dtype=params_dtype, device=device)
+        mk = lambda dt: FusedLayerNorm(kv_channels, layernorm_epsilon, apply_layernorm_1p, dtype=dt, device=device)
+        # the self-attention norms run in fp32 in the reference (promoted after load,
+        # inference/model/dit/dit_model.py:628-633); the cross-attention norms stay in bf16
+        self.q_layernorm = mk(torch.float32)
+        self.k_layernorm = mk(torch.float32)
+        self.q_layernorm_xattn = mk(params_dtype)
+        self.k_layernorm_xattn = mk(params_dtype)
+
+    # ------------------------------------------------------------------ cache
+    def _allocate_key_and_value_memory(self, sequence_length: int, batch_size: int, dtype) -> torch.Tensor:
+        """[max_seq * max_bs, Hkv, 2D] in HBM (dit_module.py:800-819; no pinned-host variant)."""
+        return torch.empty(sequence_length * batch_size, self.num_query_groups_per_partition,
+                           2 * self.hidden_size_per_attention_head, dtype=dtype,
+                           device=self.linear_qkv.q.weight.device)
+
+    def _cache(self, inference_params: InferenceParams, dtype) -> torch.Tensor:
+        d = inference_params.key_value_memory_dict
+        if self.layer_number not in d:
+            d[self.layer_number] = self._allocate_key_and_value_memory(
+                inference_params.max_sequence_length, inference_params.max_batch_size, dtype)
+        return d[self.layer_number]
+
+    # --------------------------------------------------- reference-shaped pieces
+    def _prologue_single(self, raw: torch.Tensor, which: str, cos_emb, sin_emb) -> torch.Tensor:
+        """raw [sq, b, H*D] -> [(sq b), H, D] through the fused kernel (one of q / k)."""
+        sq, b = raw.shape[0], raw.shape[1]
+        D = self.hidden_size_per_attention_head
+        flat = raw.reshape(sq * b, -1)
+        H = flat.shape[1] // D
+        rope = torch.cat([sin_emb, cos_emb], dim=-1).float().contiguous()
+        ln = self.q_layernorm if which == "q" else self.k_layernorm
+        g, be = ln.gamma_beta_fp32()
+        if which == "q":
+            q, _, _ = qk_prologue(flat, flat[:, :0], flat[:, :0], rope, g, be, None, None, Hq=H, Hkv=0, eps=self.eps,
+                                  batch=b)
+            return q
+        # K alone: run it through the Q slot (same arithmetic, contiguous output)
+        k, _, _ = qk_prologue(flat, flat[:, :0], flat[:, :0], rope, g, be, None, None, Hq=H, Hkv=0, eps=self.eps,
+                              batch=b)
+        return k
+
+    def get_q(self, mixed_qqkv: torch.Tensor, cos_emb: torch.Tensor, sin_emb: torch.Tensor) -> torch.Tensor:
+        """[sq, b, h] -> [(sq b), Hq, D]; dit_module.py:953-963."""
+        return self._prologue_single(self.linear_qkv.forward_q(mixed_qqkv), "q", cos_emb, sin_emb)
+
+    def get_k(self, mixed_qqkv: torch.Tensor, cos_emb: torch.Tensor, sin_emb: torch.Tensor) -> torch.Tensor:
+        """dit_module.py:970-980."""
+        return self._prologue_single(self.linear_qkv.forward_k(mixed_qqkv), "k", cos_emb, sin_emb)
+
+    def get_v(self, mixed_qqkv: torch.Tensor) -> torch.Tensor:
+        """dit_module.py:987-989."""
+        v = self.linear_qkv.forward_v(mixed_qqkv)
+        return v.reshape(v.shape[0] * v.shape[1], -1, self.hidden_size_per_attention_head)
+
+    def get_kv(self, mixed_qqkv: torch.Tensor, cos_emb: torch.Tensor, sin_emb: torch.Tensor) -> torch.Tensor:
+        """[(sq b), Hkv, 2D] with K | V interleaved per head; dit_module.py:991-996."""
+        _, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, want_q=False)
+        return kv
+
+    def get_qkv(self, mixed_qqkv, cos_emb, sin_emb):
+        """dit_module.py:998-1003."""
+        q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, want_q=True)
+        D = self.hidden_size_per_attention_head
+        return q, kv[..., :D].contiguous(), kv[..., D:].contiguous()
+
+    def _fused_qkv(self, mixed_qqkv, cos_emb, sin_emb, want_q=True, kv_out=None, n_cache_rows=None, kv_tail=None):
+        sq, b = mixed_qqkv.shape[0], mixed_qqkv.shape[1]
+        S = sq * b
+        Hq, Hkv = self.num_attention_heads, self.num_query_groups_per_partition
+        k_raw = self.linear_qkv.forward_k(mixed_qqkv).reshape(S, -1)
+        v_raw = self.linear_qkv.forward_v(mixed_qqkv).reshape(S, -1)
+        if want_q:
+            q_raw = self.linear_qkv.forward_q(mixed_qqkv).reshape(S, -1)
+        else:
+            q_raw = k_raw[:, :0]
+        rope = torch.cat([sin_emb, cos_emb], dim=-1).float().contiguous()
+        gq, bq = self.q_layernorm.gamma_beta_fp32()
+        gk, bk = self.k_layernorm.gamma_beta_fp32()
+        q, kv, tail = qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, Hq=Hq if want_q else 0, Hkv=Hkv,
+                                  eps=self.eps, kv_out=kv_out, n_cache_rows=n_cache_rows, kv_tail=kv_tail, batch=b)
+        return (q if want_q else None), (kv if tail is None else (kv, tail))
+
+    def get_xqkv(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor):
+        """Cross-attention q (normed) and k (normed) / v from the text states; dit_module.py:1005-1021."""
+        D = self.hidden_size_per_attention_head
+        qx = self.linear_qkv.forward_qx(mixed_qqkv)  # [sq, b, Hq*D]
+        qx = qx.transpose(0, 1).reshape(qx.shape[0] * qx.shape[1], -1, D)  # "(b sq) hn hd"
+        gq, bq = self.q_layernorm_xattn.gamma_beta_fp32()
+        qx = head_norm(qx, gq, bq, self.eps)
+        kv = torch.nn.functional.linear(key_value_states, self.linear_kv_xattn.weight)  # [Ty, 2*Hkv*D]
+        kv = kv.view(key_value_states.shape[0], -1, 2 * D)
+        gk, bk = self.k_layernorm_xattn.gamma_beta_fp32()
+        kx = head_norm(kv[..., :D], gk, bk, self.eps)  # strided read, contiguous result
+        return qx, kx, kv[..., D:]
+
+    def adjust_key_and_value_for_inference(self, key_and_value: torch.Tensor, inference_params: Optional[InferenceParams],
+                                           meta_args: ModelMetaArgs):
+        """Copying form with the reference's exact semantics (dit_module.py:891-946), for callers
+        that hold a materialised key_and_value.  forward() does not use it: it appends in place."""
+        D = self.hidden_size_per_attention_head
+        if inference_params is None:
+            return key_and_value[..., :D], key_and_value[..., D:]
+        if meta_args.extract_prefix_video_feature or meta_args.fwd_extra_1st_chunk or meta_args.slice_point > 0:
+            cache = self._cache(inference_params, key_and_value.dtype)
+            start = meta_args.slice_point * meta_args.clip_token_nums * inference_params.max_batch_size
+            prefix = cache[:start]
+            if inference_params.update_kv_cache:
+                total = key_and_value.size(0)
+                clip = (total - meta_args.clip_token_nums * inference_params.max_batch_size
+                        if meta_args.distill_nearly_clean_chunk else total)
+                if start + clip > cache.size(0):
+                    raise ValueError("KV cache overflow")
+                prefix = prefix.clone()
+                cache[start:start + clip] = key_and_value[:clip]
+            key_and_value = torch.cat([prefix, key_and_value], dim=0)
+        return key_and_value[..., :D].contiguous(), key_and_value[..., D:].contiguous()
+
+    def core_attention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, bs: int,
+                       meta_args: ModelMetaArgs) -> torch.Tensor:
+        """query [(sq b), Hq, D], key / value [(sk b), Hkv, D] -> [(sq b), Hq, D]; dit_module.py:1023-1066.
+        bs > 1 only occurs with one range per batch row (asserted there too)."""
+        p = meta_args.core_attn_params
+        if bs == 1:
+            out, _ = range_attention(query, key, value, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
+                                     return_lse=False)
+            return out
+        if meta_args.denoising_range_num > 1:
+            raise ValueError("bs > 1 with several denoising ranges is not a layout the pipeline produces")
+        out = torch.zeros_like(query)
+        sq = query.shape[0] // bs
+        one = torch.tensor([[0, sq]], dtype=torch.int32, device=query.device)
+        kone = torch.tensor([[0, key.shape[0] // bs]], dtype=torch.int32, device=query.device)
+        for b in range(bs):  # batch rows are strided views of the (sq b) token axis: no transposes
+            range_attention(query[b::bs], key[b::bs], value[b::bs], one, kone, sq, key.shape[0] // bs,
+                            out=out[b::bs], return_lse=False)
+        return out
+
+    def cross_attention(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor,
+                        cross_attn_params: PackedCrossAttnParams, get_xqkv_func: Callable) -> torch.Tensor:
+        """-> [sq, b, Hq*D]; dit_module.py:1098-1136."""
+        qx, kx, vx = get_xqkv_func(mixed_qqkv, key_value_states)
+        out, _ = range_attention(qx, kx, vx, cross_attn_params.cu_seqlens_q, cross_attn_params.cu_seqlens_kv,
+                                 cross_attn_params.max_seqlen_q, cross_attn_params.max_seqlen_kv,
+                                 ranges_mode=L.MAGI_RANGES_CU, return_lse=False)
+        b = mixed_qqkv.shape[1]
+        sq = mixed_qqkv.shape[0]
+        out = out.view(b, sq, -1)
+        return out.transpose(0, 1).contiguous() if b > 1 else out.view(sq, 1, -1)
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, hidden_states: torch.Tensor, key_value_states: torch.Tensor,
+                inference_params: Optional[InferenceParams], rotary_pos_emb: torch.Tensor, meta_args: ModelMetaArgs):
+        if rotary_pos_emb is None:
+            raise ValueError("FullyParallelAttention needs rotary_pos_emb")
+        sin_emb, cos_emb = rotary_pos_emb.tensor_split(2, -1)
+        bs = hidden_states.shape[1]
+        sq = hidden_states.shape[0]
+        D = self.hidden_size_per_attention_head
+        mixed_qqkv = self.linear_qkv.forward_ln(hidden_states)
+        p = meta_args.core_attn_params
+
+        use_cache = inference_params is not None and (
+            meta_args.extract_prefix_video_feature or meta_args.fwd_extra_1st_chunk or meta_args.slice_point > 0)
+        if not use_cache:
+            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb)
+            core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args)
+        else:
+            if bs != 1 or inference_params.max_batch_size != 1:
+                raise ValueError("the cached path runs at batch 1 (as the reference pipeline does)")
+            cache = self._cache(inference_params, hidden_states.dtype)
+            start = meta_args.slice_point * meta_args.clip_token_nums
+            S = sq
+            if inference_params.update_kv_cache:
+                n_keep = S - meta_args.clip_token_nums if meta_args.distill_nearly_clean_chunk else S
+            else:
+                n_keep = 0
+            if start + n_keep > cache.shape[0]:
+                raise ValueError("KV cache overflow")
+            tail = None
+            if n_keep < S:
+                tail = torch.empty(S - n_keep, cache.shape[1], cache.shape[2], dtype=cache.dtype, device=cache.device)
+            q, _ = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, kv_out=cache[start:], n_cache_rows=n_keep,
+                                   kv_tail=tail)
+            split = start + n_keep
+            kc, vc = cache[:split, :, :D], cache[:split, :, D:]
+            if tail is None:
+                core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
+                                          return_lse=False)
+            else:
+                core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
+                                          k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, return_lse=False)
+        core_attn_out = core.view(sq, bs, -1)
+        xattn_out = self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, self.get_xqkv)
+        return core_attn_out, xattn_out

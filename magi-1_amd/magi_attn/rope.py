@@ -1,0 +1,63 @@
+"""3-D (t, h, w) rotary table of the DiT, built on the device the caller names.
+
+Restates LearnableRotaryEmbeddingCat of the reference (inference/model/dit/dit_module.py:591-596,
+599-667, 670-717, 720-770) for its in_pixels=False use: one [S, 96] fp32 table per forward,
+[sin(48) | cos(48)], bands ordered [t(16) | h(16) | w(16)]."""
+from __future__ import annotations
+
+import math
+from typing import List, Optional, Sequence
+
+import torch
+
+
+def freq_bands(num_bands: int, temperature: float = 10000.0, step: int = 1, device=None) -> torch.Tensor:
+    exp = torch.arange(0, num_bands, step, dtype=torch.int64, device=device).to(torch.float32) / num_bands
+    return 1.0 / (temperature**exp)
+
+
+def build_rotary_table(feat_shape: Sequence[int], bands: torch.Tensor,
+                       ref_feat_shape: Optional[Sequence[float]] = None) -> torch.Tensor:
+    device = bands.device
+    axes: List[torch.Tensor] = [torch.arange(s, device=device, dtype=torch.int64).to(torch.float32) for s in feat_shape]
+    axes[1] = axes[1] - (feat_shape[1] - 1) / 2
+    axes[2] = axes[2] - (feat_shape[2] - 1) / 2
+    if ref_feat_shape is not None:
+        scaled = []
+        for x, f, r in zip(axes, feat_shape, ref_feat_shape):
+            if f == 1:
+                if r != 1:
+                    raise ValueError("ref_feat_shape must be 1 where feat_shape is 1")
+                scaled.append(x)
+            else:
+                scaled.append(x / (f - 1) * (r - 1))
+        axes = scaled
+    grid = torch.stack(torch.meshgrid(*axes, indexing="ij"), dim=-1).unsqueeze(-1)
+    pos = grid * bands
+    n = 1
+    for s in feat_shape:
+        n *= s
+    return torch.cat([pos.sin().reshape(n, -1), pos.cos().reshape(n, -1)], dim=-1)
+
+
+class LearnableRotaryEmbeddingCat(torch.nn.Module):
+    """Holds the (learnable) bands and builds the table for a [T, H, W] token grid."""
+
+    def __init__(self, dim: int, temperature: float = 10000.0, device=None):
+        super().__init__()
+        self.dim = dim
+        self.temperature = temperature
+        self.bands = torch.nn.Parameter(freq_bands(dim // 8, temperature=temperature, step=1, device=device))
+
+    def get_embed(self, shape: Sequence[int], ref_feat_shape: Optional[Sequence[float]] = None) -> torch.Tensor:
+        return build_rotary_table(shape, self.bands.detach(), ref_feat_shape)
+
+    def get_embed_for_forward(self, T: int, H: int, W: int, slice_point: int, denoising_range_num: int) -> torch.Tensor:
+        """The slice one forward consumes (inference/model/dit/dit_model.py:151-166): positions are
+        absolute in time, so the table covers the cached prefix frames too and the last T*H*W rows
+        are returned."""
+        frame_in_range = T // denoising_range_num
+        T_total = T + frame_in_range * slice_point
+        rescale = math.sqrt((H * W) / (16 * 16))
+        rope = self.get_embed([T_total, H, W], [T_total, H / rescale, W / rescale])
+        return rope[-(T * H * W):].contiguous()

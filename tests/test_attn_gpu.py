@@ -1,0 +1,234 @@
+"""GPU parity of the range-attention kernel (through the C-ABI) against the CPU oracle.
+
+Tolerance (bf16 path, from the benchmark definition): max-abs <= 2e-2 and cosine >= 0.9999
+against the fp32 reference on identical seeded inputs."""
+import numpy as np
+import pytest
+import torch
+
+import magi_attn as M
+from oracle import magi_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS = 2e-2
+MIN_COS = 0.9999
+
+
+def _cmp(out, ref, what=""):
+    o = out.detach().double().cpu().flatten()
+    r = ref.detach().double().cpu().flatten()
+    err = (o - r).abs().max().item()
+    cos = (torch.dot(o, r) / (o.norm() * r.norm()).clamp_min(1e-30)).item()
+    assert err <= MAX_ABS, f"{what}: max-abs {err}"
+    assert cos >= MIN_COS, f"{what}: cosine {cos}"
+    return err, cos
+
+
+def _ranges(dev, *arrs):
+    return [torch.tensor(np.asarray(a), dtype=torch.int32, device=dev) for a in arrs]
+
+
+CASES = [
+    # L, dn, sp, Hq, Hkv
+    (128, 1, 0, 1, 1),      # exactly one q tile, two key tiles
+    (64, 2, 0, 2, 1),       # half-filled q tile
+    (200, 3, 1, 6, 2),      # ragged everywhere, GQA 3
+    (77, 2, 2, 3, 1),       # L below one tile
+    (1, 3, 2, 6, 1),        # single-token chunks, GQA 6
+    (333, 4, 3, 12, 4),
+    (1536, 3, 0, 24, 8),    # the CPU-runnable benchmark configuration
+]
+
+
+@pytest.mark.parametrize("L,dn,sp,Hq,Hkv", CASES)
+def test_chunk_causal_parity(dev, L, dn, sp, Hq, Hkv):
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=1234 + L)
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    ref = O.range_attention(q, k, v, qr, kr)
+    lse_ref = O.range_attention_lse(q, k, v, qr, kr)
+    tq, tk = _ranges(dev, qr, kr)
+    out, lse = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, int(kr.max() - kr.min()))
+    assert out.dtype == torch.bfloat16 and out.shape == q.shape and lse.shape == (Hq, dn * L)
+    _cmp(out, ref, f"L={L}")
+    assert (lse.cpu() - lse_ref).abs().max() < 2e-3
+
+
+def test_sliding_window_ranges_and_unsorted_order(dev):
+    L, sp, dn, Hq, Hkv = 150, 8, 4, 6, 2
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=5)
+    qr = O.q_ranges_for(dn, L)
+    kr = O.noise2clean_kvrange(sp, dn, L, [5, 4, 3, 2], 1, [32, 20, 9, 0], 32)
+    perm = [2, 0, 3, 1]  # the order of the ranges must not matter
+    ref = O.range_attention(q, k, v, qr, kr)
+    tq, tk = _ranges(dev, qr[perm], kr[perm])
+    out, _ = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, 5 * L)
+    _cmp(out, ref)
+
+
+def test_empty_key_range_uncovered_rows_and_clamping(dev):
+    L, Hq, Hkv = 100, 4, 2
+    q, k, v = O.synthetic_qkv(4 * L, 3 * L, Hq, Hkv, 128, seed=6)
+    # range 0: no keys -> zeros; rows [L, 2L) in no range -> zeros (fresh output); range 2 k end past total_k -> clamped
+    qr = np.array([[0, L], [2 * L, 3 * L], [3 * L, 4 * L + 50]])
+    kr = np.array([[40, 40], [0, 2 * L], [L, 3 * L + 999]])
+    ref = O.range_attention(q, k, v, np.clip(qr, 0, 4 * L), np.clip(kr, 0, 3 * L))
+    tq, tk = _ranges(dev, qr, kr)
+    out, lse = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, L + 50, 3 * L)
+    assert torch.all(out[: 2 * L] == 0)
+    assert torch.all(torch.isinf(lse[:, :L])) and torch.all(lse[:, :L] < 0)
+    _cmp(out, ref)
+
+
+def test_many_ranges_and_q_tile_bound(dev):
+    # 40 ranges of uneven length; max_seqlen_q is only an upper bound
+    rng = np.random.default_rng(0)
+    lens = rng.integers(1, 300, size=40)
+    cu = np.concatenate([[0], np.cumsum(lens)])
+    Tq = int(cu[-1])
+    Hq, Hkv = 3, 1
+    q, k, v = O.synthetic_qkv(Tq, 700, Hq, Hkv, 128, seed=7)
+    qr = np.stack([cu[:-1], cu[1:]], 1)
+    ks = rng.integers(0, 400, size=40)
+    kr = np.stack([ks, ks + rng.integers(1, 300, size=40)], 1)
+    ref = O.range_attention(q, k, v, qr, kr)
+    tq, tk = _ranges(dev, qr, kr)
+    out, _ = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, 512, 300)
+    _cmp(out, ref)
+
+
+def test_kv_cache_views_and_two_segment_keys(dev):
+    """K / V read in place from an interleaved [T, Hkv, 2D] cache, and the key axis split into
+    [cache prefix | side buffer] must both equal attention over contiguous concatenated K / V."""
+    L, sp, dn, Hq, Hkv, D = 90, 2, 3, 6, 2, 128
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, D, seed=8)
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    ref = O.range_attention(q, k, v, qr, kr)
+    tq, tk = _ranges(dev, qr, kr)
+    cache = torch.cat([k, v], -1).to(dev)  # [T, Hkv, 2D]
+    out, _ = M.range_attention(q.to(dev), cache[..., :D], cache[..., D:], tq, tk, L)
+    _cmp(out, ref, "in-place cache")
+    base = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L)[0]
+    assert torch.equal(out, base)  # same arithmetic whatever the strides
+    for split in (0, sp * L, sp * L + 37, (sp + dn) * L):  # split inside a tile, at the ends
+        big = torch.full((split + 5, Hkv, 2 * D), float("nan"), dtype=torch.bfloat16, device=dev)
+        big[:split] = cache[:split]
+        tail = cache[split:].clone()
+        o2, _ = M.range_attention(q.to(dev), big[:split, :, :D], big[:split, :, D:], tq, tk, L,
+                                  k2=tail[..., :D], v2=tail[..., D:], k_split=split)
+        assert torch.equal(o2, base), f"split={split}"
+
+
+def test_flash_attn_func_batched_and_varlen_with_empty_segment(dev):
+    g = torch.Generator().manual_seed(9)
+    B, Sq, Sk, Hq, Hkv, D = 3, 70, 150, 4, 2, 128
+    q = torch.randn(B, Sq, Hq, D, generator=g).bfloat16()
+    k = torch.randn(B, Sk, Hkv, D, generator=g).bfloat16()
+    v = torch.randn(B, Sk, Hkv, D, generator=g).bfloat16()
+    out = M.flash_attn_func(q.to(dev), k.to(dev), v.to(dev))
+    assert out.shape == (B, Sq, Hq, D)
+    for b in range(B):
+        _cmp(out[b], O.range_attention(q[b], k[b], v[b], [[0, Sq]], [[0, Sk]]), f"batch {b}")
+    # varlen cross attention: text lengths 20..800, one empty
+    Lq = 130
+    lens = [800, 0, 20, 413]
+    qx = torch.randn(len(lens) * Lq, Hq, D, generator=g).bfloat16()
+    kx = torch.randn(sum(lens), Hkv, D, generator=g).bfloat16()
+    vx = torch.randn(sum(lens), Hkv, D, generator=g).bfloat16()
+    cu_q = torch.arange(0, (len(lens) + 1) * Lq, Lq, dtype=torch.int32)
+    cu_k = torch.tensor(np.cumsum([0] + lens), dtype=torch.int32)
+    ox = M.flash_attn_varlen_func(qx.to(dev), kx.to(dev), vx.to(dev), cu_q.to(dev), cu_k.to(dev), Lq, 800)
+    refx = O.varlen_cross_attention(qx, kx, vx, cu_q, cu_k)
+    assert torch.all(ox[Lq:2 * Lq] == 0)
+    _cmp(ox, refx)
+    with pytest.raises(NotImplementedError):
+        M.flash_attn_func(q.to(dev), k.to(dev), v.to(dev), causal=True)
+
+
+def test_softmax_scale_and_large_scores(dev):
+    # unnormalised inputs: scores of magnitude ~50 must not overflow the online softmax
+    g = torch.Generator().manual_seed(10)
+    q = (torch.randn(256, 2, 128, generator=g) * 4).bfloat16()
+    k = (torch.randn(512, 1, 128, generator=g) * 4).bfloat16()
+    v = torch.randn(512, 1, 128, generator=g).bfloat16()
+    tq, tk = _ranges(dev, [[0, 256]], [[0, 512]])
+    for scale in (None, 0.03):
+        out, _ = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, 256, softmax_scale=scale)
+        assert torch.isfinite(out).all()
+        _cmp(out, O.range_attention(q, k, v, [[0, 256]], [[0, 512]], softmax_scale=scale))
+
+
+def test_apply_rotary_emb_matches_oracle(dev):
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2, 37, 3, 128, generator=g)
+    ang = torch.randn(37, 48, generator=g)
+    cos, sin = ang.cos(), ang.sin()
+    y = M.apply_rotary_emb(x.to(dev), cos.to(dev), sin.to(dev))
+    ref = O.apply_rope_neox_partial(x, cos, sin)
+    assert (y.cpu() - ref).abs().max() < 1e-6
+    yb = M.apply_rotary_emb(x.bfloat16().to(dev), cos.to(dev), sin.to(dev))
+    assert (yb.float().cpu() - O.apply_rope_neox_partial(x.bfloat16().float(), cos, sin)).abs().max() < 2e-2
+    assert torch.equal(yb[..., 96:].cpu(), x.bfloat16()[..., 96:])
+
+
+def test_rejects_bad_arguments(dev):
+    q = torch.zeros(8, 2, 64, dtype=torch.bfloat16, device=dev)
+    r = torch.zeros(1, 2, dtype=torch.int32, device=dev)
+    with pytest.raises(M.MagiError) as e:
+        M.range_attention(q, q, q, r, r, 8)
+    assert e.value.code == -38
+    q = torch.zeros(8, 3, 128, dtype=torch.bfloat16, device=dev)
+    k = torch.zeros(8, 2, 128, dtype=torch.bfloat16, device=dev)
+    with pytest.raises(M.MagiError):
+        M.range_attention(q, k, k, r, r, 8)
+    with pytest.raises(TypeError):
+        M.range_attention(q.float(), k, k, r, r, 8)
+
+
+# ----------------------------------------------------------------------------- full-size shapes
+def _full_size_check(dev, L, dn, sp, Hq, Hkv, seed, rows_per_chunk, cpu_rows):
+    """Benchmark-size run checked on a row subsample (rows are independent, so the subsample is
+    exact): fp32 on the GPU with plain matmuls for many rows, the CPU oracle for a few."""
+    D = 128
+    g = torch.Generator(device=dev).manual_seed(seed)
+    q = torch.randn(dn * L, Hq, D, device=dev, generator=g)
+    q = (q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    cache = torch.randn((sp + dn) * L, Hkv, 2 * D, device=dev, generator=g)
+    kf = cache[..., :D]
+    cache[..., :D] = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + 1e-6)
+    cache = cache.bfloat16()
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    tq, tk = _ranges(dev, qr, kr)
+    out, lse = M.range_attention(q, cache[..., :D], cache[..., D:], tq, tk, L)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all()
+    G = Hq // Hkv
+    rs = np.random.default_rng(seed)
+    for i in range(dn):
+        rows = torch.tensor(np.sort(rs.choice(L, rows_per_chunk, replace=False)) + i * L, device=dev)
+        ke = int(kr[i, 1])
+        qs = q[rows].float()  # [r, Hq, D]
+        ref = torch.empty(rows_per_chunk, Hq, D, device=dev)
+        for hk in range(Hkv):
+            kk, vv = cache[:ke, hk, :D].float(), cache[:ke, hk, D:].float()
+            s = torch.einsum("rgd,kd->rgk", qs[:, hk * G:(hk + 1) * G], kk) * D ** -0.5
+            ref[:, hk * G:(hk + 1) * G] = torch.einsum("rgk,kd->rgd", torch.softmax(s, -1), vv)
+        _cmp(out[rows], ref, f"chunk {i} GPU fp32 subsample")
+        # a few of those rows through the CPU oracle as well
+        sub = rows[:cpu_rows].cpu()
+        o_cpu = O.range_attention(q[sub].cpu(), cache[:ke, :, :D].cpu(), cache[:ke, :, D:].cpu(), [[0, cpu_rows]], [[0, ke]])
+        _cmp(out[sub], o_cpu, f"chunk {i} CPU oracle subsample")
+        assert (ref[:cpu_rows].cpu() - o_cpu).abs().max() < 1e-4
+    # size-independent property: values all ones -> output all ones
+    ones = cache.clone()
+    ones[..., D:] = 1
+    o1, _ = M.range_attention(q, ones[..., :D], ones[..., D:], tq, tk, L, return_lse=False)
+    assert (o1.float() - 1).abs().max() <= 2 ** -7
+
+
+def test_full_size_480p_layer(dev):
+    _full_size_check(dev, 9360, 4, 4, 24, 8, seed=2234, rows_per_chunk=256, cpu_rows=8)
+
+
+def test_full_size_720p_layer(dev):
+    _full_size_check(dev, 21600, 4, 8, 48, 8, seed=3234, rows_per_chunk=128, cpu_rows=4)

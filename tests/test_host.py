@@ -1,0 +1,156 @@
+"""CPU tests of the host side: range generators and rope table of the product against the
+oracle and the reference's worked examples, the metadata builders, and the C-ABI library
+(loads, exports every declared symbol, rejects bad arguments before touching a GPU)."""
+import ctypes as C
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import magi_attn
+from magi_attn import _lib as L
+from magi_attn import params as P
+from magi_attn import ranges as R
+from magi_attn import rope as RP
+from oracle import magi_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = magi_attn.lib()
+    assert lib.magi_version() >= 100
+    header = open(os.path.join(ROOT, "include", "magi_attn.h")).read()
+    declared = set(re.findall(r"\b(magi_[a-z0-9_]+)\s*\(", header))
+    assert declared == set(L.EXPORTS), declared ^ set(L.EXPORTS)
+    for name in declared:
+        assert hasattr(lib, name), name
+
+
+def test_struct_layouts_match_header(tmp_path):
+    """ctypes mirrors vs the C compiler's view of include/magi_attn.h (sizes and field offsets)."""
+    import subprocess
+
+    fields_a = [f[0] for f in L.AttnArgs._fields_]
+    fields_p = [f[0] for f in L.PrologueArgs._fields_]
+    src = ['#include <stdio.h>', '#include <stddef.h>', '#include "magi_attn.h"', 'int main(void){',
+           'printf("%zu\\n", sizeof(magi_attn_args));']
+    src += ['printf("%%zu\\n", offsetof(magi_attn_args, %s));' % f for f in fields_a]
+    src += ['printf("%zu\\n", sizeof(magi_prologue_args));']
+    src += ['printf("%%zu\\n", offsetof(magi_prologue_args, %s));' % f for f in fields_p]
+    src += ['return 0;}']
+    c = tmp_path / "layout.c"
+    c.write_text("\n".join(src))
+    exe = tmp_path / "layout"
+    subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(c), "-o", str(exe)], check=True)
+    out = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
+    na = len(fields_a)
+    assert out[0] == C.sizeof(L.AttnArgs)
+    assert out[1:1 + na] == [getattr(L.AttnArgs, f).offset for f in fields_a]
+    assert out[1 + na] == C.sizeof(L.PrologueArgs)
+    assert out[2 + na:] == [getattr(L.PrologueArgs, f).offset for f in fields_p]
+
+
+def test_attn_argument_validation_without_gpu():
+    lib = magi_attn.lib()
+    a = L.AttnArgs()
+    a.D, a.Hq, a.Hkv = 64, 4, 2
+    assert lib.magi_attn_fwd(C.byref(a), None) == -38  # head_dim not implemented
+    assert b"head_dim" in lib.magi_last_error()
+    a.D, a.Hq, a.Hkv = 128, 5, 2
+    assert lib.magi_attn_fwd(C.byref(a), None) == -22
+    a.Hq = 4
+    a.dtype = 7
+    assert lib.magi_attn_fwd(C.byref(a), None) == -22
+    a.dtype = 0
+    a.n_ranges = 0
+    assert lib.magi_attn_fwd(C.byref(a), None) == 0  # nothing to do
+    a.n_ranges, a.total_q, a.max_seqlen_q = 1, 8, 8
+    assert lib.magi_attn_fwd(C.byref(a), None) == -22  # NULL q
+    assert b"NULL" in lib.magi_last_error()
+    a.q = a.out = a.q_ranges = a.k_ranges = 4096
+    a.q_stride_t = a.o_stride_t = 512
+    a.q_stride_h = a.o_stride_h = 128
+    a.k_stride_t, a.k_stride_h, a.v_stride_t, a.v_stride_h = 256, 128, 256, 100
+    assert lib.magi_attn_fwd(C.byref(a), None) == -22  # misaligned stride
+    assert lib.magi_attn_fwd(None, None) == -22
+
+
+def test_prologue_argument_validation_without_gpu():
+    lib = magi_attn.lib()
+    p = L.PrologueArgs()
+    p.D = 64
+    assert lib.magi_qk_prologue(C.byref(p), None) == -38
+    p.D, p.S = 128, 0
+    assert lib.magi_qk_prologue(C.byref(p), None) == 0
+    p.S, p.Hq, p.Hkv, p.R2 = 4, 2, 1, 44
+    assert lib.magi_qk_prologue(C.byref(p), None) == -22 and b"R2" in lib.magi_last_error()
+    p.R2 = 48
+    assert lib.magi_qk_prologue(C.byref(p), None) == -22  # NULL buffers
+    assert lib.magi_head_norm(None, 0, 0, None, None, None, 4, 2, 128, 0, 1e-6, None) == -22
+    assert lib.magi_apply_rotary(None, None, None, None, 1, 4, 2, 128, 80, 0, None) == -22
+
+
+def test_generate_sequences_reference_examples_and_oracle():
+    assert R.generate_sequences(8, 4, 2) == ([2, 2, 2, 2, 3, 4, 5, 6, 7], [3, 4, 5, 6, 7, 8, 8, 8, 8],
+                                             [0, 0, 0, 0, 0, 0, 1, 2, 3], [1, 2, 3, 4, 4, 4, 4, 4, 4])
+    for args in [(8, 8, 0), (8, 4, 0), (8, 1, 0), (12, 4, 3), (5, 7, 1), (1, 1, 0)]:
+        assert R.generate_sequences(*args) == O.generate_sequences(*args)
+
+
+def test_kvrange_generators_match_oracle():
+    L_ = 9360
+    for sp, dn in [(0, 1), (0, 4), (4, 4), (8, 4), (3, 2)]:
+        assert np.array_equal(R.generate_default_kvrange(sp, dn, L_).numpy(), O.default_kvrange(sp, dn, L_))
+        steps = [32, 17, 8, 0][:dn]
+        a = R.generate_noise2clean_kvrange(sp, dn, L_, [5, 4, 3, 2], 1, steps, 32).numpy()
+        assert np.array_equal(a, O.noise2clean_kvrange(sp, dn, L_, [5, 4, 3, 2], 1, steps, 32))
+        assert a.dtype == np.int32
+        b = R.generate_kvrange_for_denoising_video(sp, dn, L_, [], -1, steps, 32).numpy()
+        assert np.array_equal(b, O.default_kvrange(sp, dn, L_))
+    assert np.array_equal(R.generate_kvrange_for_prefix_video(5, L_, 1).numpy(), O.prefix_video_kvrange(5, L_, 1))
+    assert np.array_equal(R.generate_kvrange_for_prefix_video(5, L_, -1, [5, 4, 3, 2]).numpy(),
+                          O.prefix_video_kvrange(5, L_, -1, [5, 4, 3, 2]))
+    assert np.array_equal(R.generate_kv_range_for_uncondition(4, L_).numpy(), O.uncondition_kvrange(4, L_))
+    assert np.array_equal(R.q_ranges_from_chunks(4, L_).numpy(), O.q_ranges_for(4, L_))
+    # batch > 1 offsets every row by b * range_num chunks (video_generate.py:461-463)
+    two = R.generate_default_kvrange(1, 2, 10, batch_size=2).tolist()
+    assert two == [[0, 20], [0, 30], [30, 50], [30, 60]]
+    with pytest.raises(ValueError):
+        R.generate_noise2clean_kvrange(0, 2, 10, [5, 4, 3], 1, [0, 0], 32)
+
+
+def test_rope_module_matches_oracle():
+    m = RP.LearnableRotaryEmbeddingCat(128)
+    assert torch.equal(m.bands.detach(), O.freq_bands(16))
+    for T, H, W, sp, dn in [(6, 4, 6, 2, 3), (2, 16, 16, 0, 1), (4, 8, 13, 5, 2)]:
+        a = m.get_embed_for_forward(T, H, W, sp, dn)
+        b = O.rope_for_forward(T, H, W, sp, dn)
+        assert a.shape == (T * H * W, 96) and torch.equal(a, b)
+    assert torch.equal(m.get_embed([3, 4, 6]), O.rope_table(3, 4, 6))
+
+
+def test_param_builders():
+    qr = torch.tensor([[0, 10], [10, 20]], dtype=torch.int32)
+    kr = torch.tensor([[20, 50], [10, 60]], dtype=torch.int32)
+    p = P.build_core_attn_params(qr, kr, 10)
+    assert p.max_seqlen_k == 50 and p.max_seqlen_q == 10 and p.np_k_range.tolist() == kr.tolist()
+    mask = torch.zeros(3, 1, 1, 16)
+    mask[0, ..., :7] = 1
+    mask[2, ..., :3] = 1
+    x = P.build_cross_attn_params(mask, 10, 800)
+    cq, ck, qr2, kr2 = O.cross_attn_params_from_mask(mask.reshape(3, 16), 10)
+    assert torch.equal(x.cu_seqlens_q, cq) and torch.equal(x.cu_seqlens_kv, ck)
+    assert torch.equal(x.q_ranges, qr2) and torch.equal(x.kv_ranges, kr2)
+    assert x.cu_seqlens_q.dtype == torch.int32 and x.max_seqlen_kv == 800
+    ip = P.InferenceParams(1, 100)
+    assert ip.key_value_memory_dict == {} and ip.update_kv_cache is False
+
+
+def test_functional_rejects_cpu_tensors():
+    q = torch.zeros(4, 2, 128, dtype=torch.bfloat16)
+    r = torch.zeros(1, 2, dtype=torch.int32)
+    with pytest.raises(ValueError):
+        magi_attn.range_attention(q, q, q, r, r, 4)

@@ -1,0 +1,232 @@
+"""GPU parity of the fused prologue and of the module-level layer against the CPU oracle.
+
+The prologue computes in fp32 and rounds once to bf16, like the reference; summation order
+inside the norm differs from the CPU library routine, so a value that lands on a bf16 rounding
+boundary may differ by one bf16 ulp.  Bar: every element within one bf16 ulp of the oracle
+(absolute floor 1e-5 where the rotation cancels) and fewer than 1 in 1000 elements different at all."""
+import numpy as np
+import pytest
+import torch
+
+import magi_attn as M
+from magi_attn import module as MOD
+from magi_attn import params as P
+from magi_attn import ranges as R
+from oracle import magi_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _ulp_check(a, ref, what=""):
+    a, ref = a.cpu(), ref.cpu()
+    af, rf = a.float(), ref.float()
+    # one bf16 ulp of the reference value; where the rotation cancels to ~0 the fp32 rounding of the
+    # O(1) operands (~1e-6) exceeds an ulp of the tiny result, hence the absolute floor
+    ulp = torch.clamp(rf.abs() * 2.0 ** -7, min=1e-5)
+    assert torch.all((af - rf).abs() <= ulp), f"{what}: more than one bf16 ulp off"
+    frac = (a != ref).float().mean().item()
+    assert frac < 1e-3, f"{what}: {frac:.2e} of the elements differ"
+
+
+def _inputs(S, Hq, Hkv, seed):
+    g = torch.Generator().manual_seed(seed)
+    D = 128
+    qr = torch.randn(S, Hq * D, generator=g).bfloat16()
+    kr = torch.randn(S, Hkv * D, generator=g).bfloat16()
+    vr = torch.randn(S, Hkv * D, generator=g).bfloat16()
+    par = [torch.randn(D, generator=g) * 0.2 for _ in range(4)]
+    return qr, kr, vr, par
+
+
+@pytest.mark.parametrize("T,H,W,sp,dn,Hq,Hkv", [(2, 4, 6, 0, 1, 6, 2), (6, 5, 7, 2, 3, 24, 8), (4, 3, 3, 1, 2, 48, 8),
+                                                (2, 2, 2, 0, 2, 3, 1)])
+def test_prologue_parity(dev, T, H, W, sp, dn, Hq, Hkv):
+    S, D = T * H * W, 128
+    qr, kr, vr, (gq, bq, gk, bk) = _inputs(S, Hq, Hkv, seed=S + Hq)
+    rope = O.rope_for_forward(T, H, W, sp, dn)
+    q_ref, kv_ref = O.prologue(qr.view(S, Hq, D), kr.view(S, Hkv, D), vr.view(S, Hkv, D), rope, gq, bq, gk, bk)
+    to = lambda t: t.to(dev)
+    q, kv, _ = M.qk_prologue(to(qr), to(kr), to(vr), to(rope), to(gq), to(bq), to(gk), to(bk), Hq=Hq, Hkv=Hkv)
+    _ulp_check(q, q_ref, "q")
+    _ulp_check(kv[..., :D], kv_ref[..., :D], "k")
+    assert torch.equal(kv[..., D:].cpu(), kv_ref[..., D:])  # V is a copy: bit exact
+
+
+def test_prologue_rmsnorm_no_rope_and_strided_inputs(dev):
+    S, Hq, Hkv, D = 50, 6, 2, 128
+    qr, kr, vr, (gq, bq, gk, bk) = _inputs(S, Hq, Hkv, seed=3)
+    z = torch.zeros(D)
+    # one fused projection output [S, (Hq + 2 Hkv) * D] sliced into q / k / v column blocks
+    fused = torch.cat([qr, kr, vr], 1).to(dev)
+    qv, kv_, vv = fused[:, : Hq * D], fused[:, Hq * D:(Hq + Hkv) * D], fused[:, (Hq + Hkv) * D:]
+    q, kv, _ = M.qk_prologue(qv, kv_, vv, None, gq.to(dev), None, gk.to(dev), None, Hq=Hq, Hkv=Hkv,
+                             norm_kind=M.MAGI_NORM_RMSNORM_1P)
+    q_ref = O.rmsnorm(qr.view(S, Hq, D).float(), gq + 1).bfloat16()
+    k_ref = O.rmsnorm(kr.view(S, Hkv, D).float(), gk + 1).bfloat16()
+    _ulp_check(q, q_ref, "q rms")
+    _ulp_check(kv[..., :D], k_ref, "k rms")
+    q2, _, _ = M.qk_prologue(qv, kv_, vv, None, None, None, None, None, Hq=Hq, Hkv=Hkv, norm_kind=M.MAGI_NORM_NONE)
+    assert torch.equal(q2.cpu(), qr.view(S, Hq, D))
+
+
+def test_prologue_writes_cache_in_place_and_tail(dev):
+    S, Hq, Hkv, D = 40, 3, 2, 128
+    qr, kr, vr, (gq, bq, gk, bk) = _inputs(S, Hq, Hkv, seed=4)
+    rope = O.rope_table(1, 5, 8)
+    _, kv_ref = O.prologue(qr.view(S, Hq, D), kr.view(S, Hkv, D), vr.view(S, Hkv, D), rope, gq, bq, gk, bk)
+    to = lambda t: t.to(dev)
+    cache = torch.full((100, Hkv, 2 * D), 7.0, dtype=torch.bfloat16, device=dev)
+    tail = torch.full((20, Hkv, 2 * D), 9.0, dtype=torch.bfloat16, device=dev)
+    start, keep = 30, 25
+    M.qk_prologue(to(qr), to(kr), to(vr), to(rope), to(gq), to(bq), to(gk), to(bk), Hq=Hq, Hkv=Hkv,
+                  kv_out=cache[start:], n_cache_rows=keep, kv_tail=tail)
+    assert torch.all(cache[:start] == 7) and torch.all(cache[start + keep:] == 7)  # nothing else touched
+    _ulp_check(cache[start:start + keep], kv_ref[:keep], "cache rows")
+    _ulp_check(tail[: S - keep], kv_ref[keep:], "tail rows")
+    assert torch.all(tail[S - keep:] == 9)
+
+
+def test_head_norm_matches_bf16_layernorm(dev):
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(33, 5, 256, generator=g).bfloat16()
+    w = (torch.randn(128, generator=g) * 0.1).bfloat16()
+    b = (torch.randn(128, generator=g) * 0.1).bfloat16()
+    ln = MOD.FusedLayerNorm(128, dtype=torch.bfloat16)
+    ln.weight.data.copy_(w)
+    ln.bias.data.copy_(b)
+    gg, bb = ln.gamma_beta_fp32()
+    y = M.head_norm(x.to(dev)[..., :128], gg.to(dev), bb.to(dev))  # strided K half of an interleaved KV
+    ref = torch.nn.functional.layer_norm(x[..., :128], (128,), w + 1, b, 1e-6)  # what the reference calls in bf16
+    _ulp_check(y, ref, "xattn norm")
+
+
+# ----------------------------------------------------------------------------- the layer
+def _make_layer(dev, hidden, Hq, Hkv, seed):
+    torch.manual_seed(seed)
+    layer = MOD.FullyParallelAttention(hidden, Hq, Hkv, layer_number=3, device=dev)
+    with torch.no_grad():
+        for p in layer.parameters():
+            if p.dim() == 1:
+                p.copy_(torch.randn_like(p.float()) * 0.1)
+            else:
+                p.copy_(torch.randn_like(p.float()) * hidden ** -0.5)
+        layer.linear_qkv.layer_norm.weight.add_(1.0)
+    return layer
+
+
+def _oracle_layer(layer, hidden_states, y, rope, sp, L, k_range, q_range, cache, update, distill, extra, cu_q, cu_k,
+                  has_ip=True):
+    """The reference's forward (dit_module.py:1138-1173) restated with the oracle pieces, on CPU."""
+    D = 128
+    cpu = lambda t: t.detach().cpu()
+    lq = layer.linear_qkv
+    mixed = torch.nn.functional.layer_norm(hidden_states, (hidden_states.shape[-1],), cpu(lq.layer_norm.weight),
+                                           cpu(lq.layer_norm.bias), 1e-6)
+    S = mixed.shape[0]
+    lin = lambda m: torch.nn.functional.linear(mixed[:, 0], cpu(m.weight))
+    Hq, Hkv = layer.num_attention_heads, layer.num_query_groups_per_partition
+    q_raw, k_raw, v_raw, qx_raw = lin(lq.q), lin(lq.k), lin(lq.v), lin(lq.qx)
+    q, kv = O.prologue(q_raw.view(S, Hq, D), k_raw.view(S, Hkv, D), v_raw.view(S, Hkv, D), rope,
+                       cpu(layer.q_layernorm.weight), cpu(layer.q_layernorm.bias), cpu(layer.k_layernorm.weight),
+                       cpu(layer.k_layernorm.bias))
+    k, v = cache.adjust(kv, has_inference_params=has_ip, update_kv_cache=update, slice_point=sp, clip_token_nums=L,
+                        fwd_extra_1st_chunk=extra, distill_nearly_clean_chunk=distill)
+    core = O.range_attention(q, k, v, q_range, k_range).bfloat16()
+    qx = torch.nn.functional.layer_norm(qx_raw.view(S, Hq, D), (D,), cpu(layer.q_layernorm_xattn.weight) + 1,
+                                        cpu(layer.q_layernorm_xattn.bias), 1e-6)
+    kvx = torch.nn.functional.linear(y, cpu(layer.linear_kv_xattn.weight)).view(y.shape[0], Hkv, 2 * D)
+    kx = torch.nn.functional.layer_norm(kvx[..., :D], (D,), cpu(layer.k_layernorm_xattn.weight) + 1,
+                                        cpu(layer.k_layernorm_xattn.bias), 1e-6)
+    xo = O.varlen_cross_attention(qx, kx, kvx[..., D:], cu_q, cu_k).bfloat16()
+    return core.reshape(S, 1, -1), xo.reshape(S, 1, -1)
+
+
+def test_layer_forward_sequence_with_kv_cache(dev):
+    """A short generation schedule (clean-chunk extraction, cached denoising with and without cache
+    update, nearly-clean distillation, a cache-less pass) through the layer, compared step by
+    step with the oracle's layer and with the oracle's cache contents."""
+    hidden, Hq, Hkv, D = 256, 6, 2, 128
+    fr, H, W = 2, 3, 4
+    L = fr * H * W
+    n_chunks = 6
+    layer = _make_layer(dev, hidden, Hq, Hkv, seed=0)
+    rope_mod = M.rope.LearnableRotaryEmbeddingCat(128, device=dev) if hasattr(M, "rope") else None
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+    rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
+    ip = P.InferenceParams(1, n_chunks * L)
+    cache_ref = O.KVCacheModel(n_chunks * L, Hkv, D)
+    g = torch.Generator().manual_seed(1)
+    #        sp dn update distill extra has_ip
+    steps = [(0, 2, True, False, True, True),
+             (0, 3, True, True, True, True),
+             (2, 3, False, False, False, True),
+             (2, 3, True, False, False, True),
+             (1, 4, True, True, True, True),
+             (3, 3, False, False, True, True),
+             (0, 2, False, False, False, False)]
+    for sp, dn, update, distill, extra, has_ip in steps:
+        S = dn * L
+        hs = torch.randn(S, 1, hidden, generator=g).bfloat16()
+        lens = torch.randint(0, 9, (dn,), generator=g)
+        mask = (torch.arange(8)[None] < lens[:, None]).float().view(dn, 1, 1, 8)
+        y = (torch.randn(int(lens.sum()), hidden, generator=g) * 0.5).bfloat16()
+        k_range = R.generate_default_kvrange(sp, dn, L) if has_ip else R.generate_kv_range_for_uncondition(dn, L)
+        q_range = R.q_ranges_from_chunks(dn, L)
+        core_p = P.build_core_attn_params(q_range.to(dev), k_range.to(dev), L)
+        cross_p = P.build_cross_attn_params(mask.to(dev), L, 8)
+        meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=sp, denoising_range_num=dn,
+                               range_num=sp + dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=extra,
+                               distill_nearly_clean_chunk=distill, clip_token_nums=L, enable_cuda_graph=False,
+                               core_attn_params=core_p, cross_attn_params=cross_p)
+        rope = rope_mod.get_embed_for_forward(dn * fr, H, W, sp, dn)
+        ip.update_kv_cache = update
+        with torch.no_grad():
+            core, xo = layer(hs.to(dev), y.to(dev), ip if has_ip else None, rope, meta)
+        assert core.shape == (S, 1, Hq * D) and xo.shape == (S, 1, Hq * D)
+        core_ref, xo_ref = _oracle_layer(layer, hs, y, O.rope_for_forward(dn * fr, H, W, sp, dn), sp, L,
+                                         k_range.numpy(), q_range.numpy(), cache_ref, update, distill, extra,
+                                         cross_p.cu_seqlens_q.cpu(), cross_p.cu_seqlens_kv.cpu(), has_ip)
+        for a, b, nm in ((core, core_ref, "core"), (xo, xo_ref, "xattn")):
+            err = (a.float().cpu() - b.float()).abs().max().item()
+            assert err <= 3e-2, f"step {(sp, dn, update, distill, extra)} {nm}: {err}"
+        # what the cache holds afterwards must be what the reference's cache would hold
+        if has_ip and (extra or sp > 0) and update:
+            keep = S - L if distill else S
+            got = ip.key_value_memory_dict[3][sp * L: sp * L + keep].float().cpu()
+            want = cache_ref.mem[sp * L: sp * L + keep].float()
+            assert (got - want).abs().max() <= 3e-2
+
+
+def test_layer_batched_cacheless_pass(dev):
+    """The unconditional pass of classifier-free guidance: chunks become batch rows, tokens are
+    ordered (position, batch), every row attends to itself only, no cache."""
+    hidden, Hq, Hkv, D = 256, 6, 2, 128
+    fr, H, W, B = 2, 3, 4, 3
+    L = fr * H * W
+    layer = _make_layer(dev, hidden, Hq, Hkv, seed=2)
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+    rope = LearnableRotaryEmbeddingCat(128, device=dev).get_embed_for_forward(fr, H, W, 0, 1)
+    g = torch.Generator().manual_seed(3)
+    hs = torch.randn(L, B, hidden, generator=g).bfloat16()
+    lens = torch.tensor([3, 0, 8])
+    mask = (torch.arange(8)[None] < lens[:, None]).float().view(B, 1, 1, 8)
+    y = (torch.randn(int(lens.sum()), hidden, generator=g) * 0.5).bfloat16()
+    k_range = R.generate_kv_range_for_uncondition(B, L)
+    core_p = P.build_core_attn_params(k_range.to(dev), k_range.to(dev), L)
+    cross_p = P.build_cross_attn_params(mask.to(dev), L, 8)
+    meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=0, denoising_range_num=1,
+                           range_num=1, extract_prefix_video_feature=False, fwd_extra_1st_chunk=False,
+                           distill_nearly_clean_chunk=False, clip_token_nums=L, enable_cuda_graph=False,
+                           core_attn_params=core_p, cross_attn_params=cross_p)
+    with torch.no_grad():
+        core, xo = layer(hs.to(dev), y.to(dev), None, rope, meta)
+    assert core.shape == (L, B, Hq * D)
+    cu_k = cross_p.cu_seqlens_kv.cpu()
+    for b in range(B):  # each batch row == a batch-1 forward of that row
+        cache_ref = O.KVCacheModel(L, Hkv, D)
+        yb = y[cu_k[b]:cu_k[b + 1]]
+        c_ref, x_ref = _oracle_layer(layer, hs[:, b:b + 1], yb, O.rope_for_forward(fr, H, W, 0, 1), 0, L,
+                                     np.array([[0, L]]), np.array([[0, L]]), cache_ref, False, False, False,
+                                     torch.tensor([0, L]), torch.tensor([0, int(lens[b])]), has_ip=False)
+        assert (core[:, b].float().cpu() - c_ref[:, 0].float()).abs().max() <= 3e-2
+        assert (xo[:, b].float().cpu() - x_ref[:, 0].float()).abs().max() <= 3e-2

@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A step is one layer-forward of the path on the 720p 24B-style shape: fused prologue
+(QK-LayerNorm + 3-D RoPE + bf16 cast + in-place KV-cache append) -> chunk-causal range
+attention over [8 cached prefix chunks | 4 denoising chunks] -> T5 cross-attention (two head
+norms + varlen attention).  Inputs are synthetic, seeded, and resident in HBM before the
+timed region.  One JSON line is printed; `value` is the masked-corrected attention TFLOP/s of
+the whole step (core + cross attention FLOPs over the step's wall time), `roofline` prices the
+dominant kernel (core attention) against the MI355X dense bf16 MFMA peak from HIP-event
+timings of that kernel alone, and `cpu_baseline` times the CPU oracle (torch SDPA fp32, same
+ranges) on a bounded sample of the same workload on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "magi-1_amd"))
+
+import numpy as np
+import torch
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_FP8_TFLOPS = 5000.0
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (T_lat frames per chunk, H, W, denoise chunks, prefix chunks, Hq, Hkv)
+    "720p-24B": (6, 45, 80, 4, 8, 48, 8),
+    "480p-4.5B": (6, 30, 52, 4, 4, 24, 8),
+}
+
+
+def build_inputs(name, dev, seed=1234):
+    import magi_attn as M
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+
+    fr, H, W, dn, sp, Hq, Hkv = WORKLOADS[name]
+    D = 128
+    L = fr * H * W
+    S = dn * L
+    g = torch.Generator(device=dev).manual_seed(seed + 2000)
+    rn = lambda *shape: torch.randn(*shape, device=dev, generator=g).bfloat16()
+    rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
+    zeros = torch.zeros(D, device=dev)
+    # KV cache for the whole window, prefix filled by the same prologue (clean chunks, same distribution)
+    cache = torch.empty((sp + dn) * L, Hkv, 2 * D, dtype=torch.bfloat16, device=dev)
+    for c0 in range(0, sp, 4):
+        n = min(4, sp - c0)
+        rope_p = rope_mod.get_embed_for_forward(n * fr, H, W, c0, n)
+        k_raw, v_raw = rn(n * L, Hkv * D), rn(n * L, Hkv * D)
+        M.qk_prologue(k_raw[:, :0], k_raw, v_raw, rope_p, None, None, zeros, zeros, Hq=0, Hkv=Hkv,
+                      kv_out=cache[c0 * L:], n_cache_rows=n * L)
+    inp = dict(
+        name=name, L=L, S=S, dn=dn, sp=sp, Hq=Hq, Hkv=Hkv, D=D, cache=cache, zeros=zeros,
+        q_raw=rn(S, Hq * D), k_raw=rn(S, Hkv * D), v_raw=rn(S, Hkv * D), qx_raw=rn(S, Hq, D),
+        rope=rope_mod.get_embed_for_forward(dn * fr, H, W, sp, dn),
+        q=torch.empty(S, Hq, D, dtype=torch.bfloat16, device=dev),
+        out=torch.empty(S, Hq, D, dtype=torch.bfloat16, device=dev),
+        xout=torch.empty(S, Hq, D, dtype=torch.bfloat16, device=dev),
+    )
+    from magi_attn import ranges as R
+
+    inp["q_ranges"] = R.q_ranges_from_chunks(dn, L, device=dev)
+    inp["k_ranges"] = R.generate_default_kvrange(sp, dn, L, device=dev)
+    # T5 side: valid lengths uniform in [20, 800] per chunk, K | V interleaved per head as the projection emits them
+    rs = np.random.default_rng(seed)
+    lens = rs.integers(20, 801, size=dn)
+    inp["t5_lens"] = lens
+    inp["cu_q"] = torch.arange(0, (dn + 1) * L, L, dtype=torch.int32, device=dev)
+    inp["cu_k"] = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32, device=dev)
+    inp["kvx"] = rn(int(lens.sum()), Hkv, 2 * D)
+    return inp
+
+
+def flops_of(inp):
+    L, dn, sp, Hq, D = inp["L"], inp["dn"], inp["sp"], inp["Hq"], inp["D"]
+    core = 4.0 * D * Hq * sum(L * (sp + j + 1) * L for j in range(dn))
+    cross = 4.0 * D * Hq * float(sum(L * int(n) for n in inp["t5_lens"]))
+    return core, cross
+
+
+def prologue_bytes(inp):
+    S, Hq, Hkv, D = inp["S"], inp["Hq"], inp["Hkv"], inp["D"]
+    return 2 * (S * Hq * D * 2) + 2 * (S * Hkv * 2 * D * 2) + S * 96 * 4
+
+
+def run_step(inp, ev=None):
+    """One layer-forward of the hot path.  ev: optional dict of event pairs to record around kernels."""
+    import magi_attn as M
+
+    L, sp, D = inp["L"], inp["sp"], inp["D"]
+    cache = inp["cache"]
+    z = inp["zeros"]
+
+    def rec(key, which):
+        if ev is not None:
+            ev[key][which].record()
+
+    rec("prologue", 0)
+    M.qk_prologue(inp["q_raw"], inp["k_raw"], inp["v_raw"], inp["rope"], z, z, z, z, Hq=inp["Hq"], Hkv=inp["Hkv"],
+                  kv_out=cache[sp * L:], n_cache_rows=inp["S"], q_out=inp["q"])
+    rec("prologue", 1)
+    rec("core", 0)
+    M.range_attention(inp["q"], cache[..., :D], cache[..., D:], inp["q_ranges"], inp["k_ranges"], L,
+                      out=inp["out"], return_lse=False)
+    rec("core", 1)
+    rec("cross", 0)
+    qx = M.head_norm(inp["qx_raw"], z, z)
+    kx = M.head_norm(inp["kvx"][..., :D], z, z)
+    M.range_attention(qx, kx, inp["kvx"][..., D:], inp["cu_q"], inp["cu_k"], L, 800, ranges_mode=M.MAGI_RANGES_CU,
+                      out=inp["xout"], return_lse=False)
+    rec("cross", 1)
+
+
+def cpu_baseline(inp, rows_per_chunk=6144):
+    """CPU oracle (torch SDPA fp32, one call per range) on a bounded sample of the workload:
+    the first rows_per_chunk queries of every denoising chunk, the 6 (= Hq/Hkv) q heads of KV
+    head 0, full key ranges.  Heads and rows are independent, so this is a slice of the real job."""
+    from oracle import magi_oracle as O
+
+    L, dn, sp, Hq, Hkv, D = inp["L"], inp["dn"], inp["sp"], inp["Hq"], inp["Hkv"], inp["D"]
+    G = Hq // Hkv
+    rows = min(rows_per_chunk, L)
+    idx = torch.cat([torch.arange(j * L, j * L + rows) for j in range(dn)])
+    q = inp["q"][idx.to(inp["q"].device), :G].float().cpu()
+    k = inp["cache"][:, :1, :D].float().cpu()
+    v = inp["cache"][:, :1, D:].float().cpu()
+    qr = np.array([[j * rows, (j + 1) * rows] for j in range(dn)])
+    kr = np.array([[0, (sp + j + 1) * L] for j in range(dn)])
+    fl = O.attention_flops(qr, kr, G, D)
+    torch.set_num_threads(os.cpu_count() if os.cpu_count() and os.cpu_count() <= 64 else torch.get_num_threads())
+    t0 = time.perf_counter()
+    o = O.range_attention(q, k, v, qr, kr)
+    dt = time.perf_counter() - t0
+    return dict(value=fl / dt / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"first {rows} q rows of each of the {dn} chunks x {G} q heads of kv head 0, full key ranges, "
+                       f"{fl:.3e} FLOP in {dt:.1f} s (torch {torch.__version__} CPU SDPA fp32)"), o, idx
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="720p-24B", choices=sorted(WORKLOADS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(2)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    inp = build_inputs(args.workload, dev)
+    core_fl, cross_fl = flops_of(inp)
+
+    for _ in range(args.warmup):
+        run_step(inp)
+    torch.cuda.synchronize()
+    keys = ("prologue", "core", "cross")
+    evs = [{k: (torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for k in keys}
+           for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for s in range(args.steps):
+        run_step(inp, evs[s])
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    kern_ms = {k: float(np.mean([e[k][0].elapsed_time(e[k][1]) for e in evs])) for k in keys}
+
+    value = (core_fl + cross_fl) / (ms_per_step * 1e-3) / 1e12
+    core_tflops = core_fl / (kern_ms["core"] * 1e-3) / 1e12
+    pro_gbs = prologue_bytes(inp) / (kern_ms["prologue"] * 1e-3) / 1e9
+    result = {
+        "metric": "attention TFLOP/s (masked-corrected), chunk-causal layer, 1 GPU",
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload} layer-forward: prologue + chunk-causal attention "
+                               f"(Q {inp['S']} tok x {inp['Hq']} heads over K/V {(inp['sp'] + inp['dn']) * inp['L']} tok x "
+                               f"{inp['Hkv']} heads, d=128, {inp['sp']} cached + {inp['dn']} denoising chunks of {inp['L']}) "
+                               f"+ T5 cross-attention (lens {inp['t5_lens'].tolist()})",
+                   "core_flops": core_fl, "cross_flops": cross_fl},
+        "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_kernel", "achieved": round(core_tflops, 2),
+                     "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(core_tflops / PEAK_BF16_TFLOPS, 4),
+                     "traffic": None, "ms": round(kern_ms["core"], 3)},
+        "roofline_prologue": {"bound": "hbm", "kernel": "prologue_kernel", "achieved": round(pro_gbs, 1),
+                              "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(pro_gbs / PEAK_HBM_GBS, 4),
+                              "traffic": None, "ms": round(kern_ms["prologue"], 4)},
+        "cross_attention_ms": round(kern_ms["cross"], 4),
+    }
+    if not args.no_cpu_baseline:
+        cb, o_cpu, idx = cpu_baseline(inp)
+        got = inp["out"][idx.to(dev), : inp["Hq"] // inp["Hkv"]].float().cpu()
+        cb["max_abs_vs_gpu"] = round((got - o_cpu).abs().max().item(), 5)
+        result["cpu_baseline"] = cb
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -3,6 +3,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 
 #include "kernels.h"
@@ -100,7 +101,11 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.k_split = k_split;
   a.n_ranges = p->n_ranges;
   a.ranges_mode = p->ranges_mode;
-  a.tiles_per_range = (p->max_seqlen_q + magi::kAttnBlockM - 1) / magi::kAttnBlockM;
+  a.block_m = 128;
+  if (const char* e = std::getenv("MAGI_ATTN_BLOCK_M")) {  // tuning knob: 128 or 256
+    if (std::atoi(e) == 256) a.block_m = 256;
+  }
+  a.tiles_per_range = (p->max_seqlen_q + a.block_m - 1) / a.block_m;
   a.Hq = p->Hq;
   a.Hkv = p->Hkv;
   a.G = p->Hq / p->Hkv;

@@ -1,7 +1,8 @@
 // Range attention forward, bf16 in / bf16 out, fp32 online softmax, for gfx950 (MI355X).
 //
-// One workgroup = 4 wavefronts = 128 query rows of one (range, q head); wave w owns rows
-// 32w..32w+31.  Key/value rows stream through LDS in tiles of 64, double buffered.
+// One workgroup = NW wavefronts = 32*NW query rows of one (range, q head); wave w owns rows
+// 32w..32w+31.  Key/value rows stream through LDS in tiles of 64, double buffered, filled by
+// direct global->LDS loads (no register staging).
 //
 // The scores are computed transposed, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: the
 // accumulator layout then puts ONE query per lane column (lane % 32) and spreads the keys over
@@ -9,6 +10,12 @@
 // the two half-waves, and the probabilities are already in the B-operand layout of the second
 // product O^T = V^T P^T.  V^T is fetched from the row-major V tile with the transposing LDS
 // read ds_read_b64_tr_b16.
+//
+// LDS tile layout: 64 rows of 256 bytes; the 16-byte chunk c of row r lives at chunk
+// c ^ (r & 15) for K (conflict-free ds_read_b128 down a column of rows) and at
+// c ^ ((r & 3) << 2) for V (conflict-free transposing reads of 4-row groups).  A direct load
+// places lane l's 16 bytes at base + 16*l, so the swizzle is applied on the global side: lane
+// l fetches the logical chunk that belongs at its fixed LDS slot.
 //
 // Work decomposition: blockIdx -> (kv head, range slot, q tile, q head within the GQA group),
 // laid out so that the workgroups an XCD receives (blockIdx % 8) share a KV head and walk the
@@ -29,10 +36,10 @@ typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
 #define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
+#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
-constexpr int BM = kAttnBlockM;  // q rows per workgroup
-constexpr int BN = 64;           // keys per tile
-constexpr int ROW_BYTES = 256;   // D = 128 bf16
+constexpr int BN = 64;          // keys per tile
+constexpr int ROW_BYTES = 256;  // D = 128 bf16
 constexpr int TILE_BYTES = BN * ROW_BYTES;
 constexpr int MAX_SORT = 256;
 
@@ -54,8 +61,11 @@ __device__ __forceinline__ void load_range(const int* r, int mode, int i, int to
   e = max(s, min(e, total));
 }
 
-__global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
-  __shared__ __attribute__((aligned(16))) unsigned char smem[2][2][TILE_BYTES];  // [buffer][K|V]
+template <int NW>
+__global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
+  constexpr int BM = 32 * NW;
+  constexpr int LOADS = 16 / NW;  // direct loads per wave per matrix per tile (4 rows each)
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[2][2][TILE_BYTES];  // [buffer][K|V]
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -90,7 +100,7 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const At
       if (rank == (int)rslot) s_sel = tid;
     }
     __syncthreads();
-    ridx = s_sel;
+    ridx = __builtin_amdgcn_readfirstlane(s_sel);
   } else {
     ridx = a.n_ranges - 1 - (int)rslot;
   }
@@ -100,7 +110,8 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const At
   const int q0 = qs + (int)tile * BM;
   if (q0 >= qe) return;
 
-  const int w = tid >> 6, l = tid & 63, i = l & 31, g = l >> 5;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l = tid & 63, i = l & 31, g = l >> 5;
   const int q_row = q0 + 32 * w + i;
   const bool row_ok = q_row < qe;
 
@@ -123,37 +134,46 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const At
     for (int kk = 0; kk < 8; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 32);
   }
 
-  // ---- K/V tile movers: thread owns 16-byte column chunk cc of rows r0 + 16j ----
-  const int cc = tid & 15, r0 = tid >> 4;
-  const long kcol = (long)kvh * a.ks_h + cc * 16;
-  const long vcol = (long)kvh * a.vs_h + cc * 16;
-  const int st_k = r0 * ROW_BYTES + ((cc ^ r0) << 4);               // K tile: chunk ^= row & 15
-  const int st_v = r0 * ROW_BYTES + ((cc ^ ((r0 & 3) << 2)) << 4);  // V tile: chunk ^= (row & 3) << 2
-  u32x4 kr[4], vr[4];
-
-  // rows >= k_split come from the second segment: same strides, so only the base differs
-  const char* const kbase = a.k;
-  const char* const vbase = a.v;
-  const long k2_delta = a.k2 ? (a.k2 - a.k) - (long)a.k_split * a.ks_t : 0;
-  const long v2_delta = a.v2 ? (a.v2 - a.v) - (long)a.k_split * a.vs_t : 0;
-  const int k_split = a.k_split;
+  // ---- K/V tile loader: wave w fills rows 4*(w + NW*j) .. +3; lane l sits at row +(l >> 4), slot l & 15 ----
+  const int lrow = l >> 4, slot = l & 15;
+  const int row_in_tile0 = 4 * w + lrow;                    // + 4*NW*j
+  const int kchunk = slot ^ ((4 * (w & 3) + lrow) & 15);    // logical chunk that belongs in this K slot
+  const int vchunk = slot ^ (lrow << 2);                    // ... in this V slot
   const long ks_t = a.ks_t, vs_t = a.vs_t;
-  auto fetch = [&](int k0) {
+  const int k_split = a.k_split;
+  const long k2_delta = a.k2 ? (a.k2 - a.k) - (long)k_split * ks_t : 0;
+  const long v2_delta = a.v2 ? (a.v2 - a.v) - (long)k_split * vs_t : 0;
+  const char* const kcolp = a.k + (long)kvh * a.ks_h;
+  const char* const vcolp = a.v + (long)kvh * a.vs_h;
+  const unsigned kvoff = (unsigned)row_in_tile0 * (unsigned)ks_t + (unsigned)(kchunk * 16);
+  const unsigned vvoff = (unsigned)row_in_tile0 * (unsigned)vs_t + (unsigned)(vchunk * 16);
+  const bool small_strides = ks_t * (BN + 4) < (1l << 31) && vs_t * (BN + 4) < (1l << 31);
+
+  auto issue_tile = [&](int k0, int buf) {
+    unsigned char* kdst = &smem[buf][0][w * 1024];
+    unsigned char* vdst = &smem[buf][1][w * 1024];
+    const bool interior = small_strides && (k0 + BN <= ke) && (k0 + BN <= k_split || k0 >= k_split);
+    if (interior) {  // uniform base + per-lane 32-bit offset
+      const bool second = k0 >= k_split;
+      const char* kb = kcolp + (long)k0 * ks_t + (second ? k2_delta : 0);
+      const char* vb = vcolp + (long)k0 * vs_t + (second ? v2_delta : 0);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int row = min(k0 + r0 + 16 * j, ke - 1);
-      const bool second = row >= k_split;
-      const long ko = (long)row * ks_t + kcol + (second ? k2_delta : 0);
-      const long vo = (long)row * vs_t + vcol + (second ? v2_delta : 0);
-      kr[j] = *(const u32x4*)(kbase + ko);
-      vr[j] = *(const u32x4*)(vbase + vo);
-    }
-  };
-  auto stash = [&](int buf) {
+      for (int j = 0; j < LOADS; ++j) {
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kb + (long)(4 * NW * j) * ks_t + kvoff),
+                                         LDS_PTR(void, kdst + j * NW * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vb + (long)(4 * NW * j) * vs_t + vvoff),
+                                         LDS_PTR(void, vdst + j * NW * 1024), 16, 0, 0);
+      }
+    } else {  // ragged end of the range, or a tile that straddles the two key segments
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      *LDS_PTR(u32x4, &smem[buf][0][st_k + j * 16 * ROW_BYTES]) = kr[j];
-      *LDS_PTR(u32x4, &smem[buf][1][st_v + j * 16 * ROW_BYTES]) = vr[j];
+      for (int j = 0; j < LOADS; ++j) {
+        const int row = min(k0 + row_in_tile0 + 4 * NW * j, ke - 1);
+        const bool second = row >= k_split;
+        const char* kp = kcolp + (long)row * ks_t + (second ? k2_delta : 0) + kchunk * 16;
+        const char* vp = vcolp + (long)row * vs_t + (second ? v2_delta : 0) + vchunk * 16;
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kp), LDS_PTR(void, kdst + j * NW * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vp), LDS_PTR(void, vdst + j * NW * 1024), 16, 0, 0);
+      }
     }
   };
 
@@ -174,32 +194,52 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const At
   float l_run = 0.f;                // this lane's share of the running sum
   const float c = a.scale_log2;
   const bool wave_on = (q0 + 32 * w) < qe;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   const int n_tiles = (ke - ks + BN - 1) / BN;
-  fetch(ks);
+  issue_tile(ks, 0);
   for (int it = 0; it < n_tiles; ++it) {
     const int buf = it & 1;
     const int k0 = ks + it * BN;
-    stash(buf);
-    __syncthreads();
-    if (it + 1 < n_tiles) fetch(k0 + BN);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile `it` is in LDS
+    __syncthreads();                                   // ... and everybody else's; buffer buf^1 is free
+    if (it + 1 < n_tiles) issue_tile(k0 + BN, buf ^ 1);
     if (!wave_on) continue;
 
     const unsigned char* Kt = &smem[buf][0][0];
     const unsigned char* Vt = &smem[buf][1][0];
 
-    // S^T[key][q] for 64 keys x 32 queries
+    // LDS operand fetchers
+    auto read_k = [&](int t, int kk) -> bf16x8 {
+      return *LDS_PTR(const bf16x8, Kt + ((base_k ^ (kk << 5)) + t * 32 * ROW_BYTES));
+    };
+    auto read_v = [&](int mb, int s) -> bf16x8 {
+      const int bv = base_v ^ (mb << 6);
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * s) * ROW_BYTES)));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * s + 8) * ROW_BYTES)));
+      const s16x8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8, va);
+    };
+
+    // S^T[key][q] for 64 keys x 32 queries.  Operand reads run one half-tile ahead of the MFMAs
+    // that consume them, and the first V operands are fetched under the second half's MFMAs.
     f32x16 s_acc[2];
+    bf16x8 ka[8], kb[8], vbuf[8];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
+    for (int kk = 0; kk < 8; ++kk) ka[kk] = read_k(0, kk);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int v = 0; v < 16; ++v) s_acc[t][v] = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk) {
-        const bf16x8 ka = *LDS_PTR(const bf16x8, Kt + ((base_k ^ (kk << 5)) + t * 32 * ROW_BYTES));
-        s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka, qf[kk], s_acc[t], 0, 0, 0);
-      }
+    for (int kk = 0; kk < 8; ++kk) {
+      s_acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], kk == 0 ? zero16 : s_acc[0], 0, 0, 0);
+      kb[kk] = read_k(1, kk);
     }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      s_acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kb[kk], qf[kk], kk == 0 ? zero16 : s_acc[1], 0, 0, 0);
+      vbuf[kk] = read_v(kk >> 2, kk & 3);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     if (k0 + BN > ke) {  // ragged last tile: keys >= ke do not exist
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -242,16 +282,14 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const At
         for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
     }
 
-    // O^T[d][q] += V^T[d][key] P^T[key][q]
+    // O^T[d][q] += V^T[d][key] P^T[key][q]; V operands of d-block mb + 2 are fetched while block mb multiplies
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
-      const int bv = base_v ^ (mb << 6);
 #pragma unroll
       for (int s = 0; s < 4; ++s) {
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * s) * ROW_BYTES)));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * s + 8) * ROW_BYTES)));
-        const s16x8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        o_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, va), pb[s], o_acc[mb], 0, 0, 0);
+        o_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vbuf[(mb & 1) * 4 + s], pb[s], o_acc[mb], 0, 0, 0);
+        if (mb + 2 < 4) vbuf[(mb & 1) * 4 + s] = read_v(mb + 2, s);
       }
     }
   }
@@ -281,7 +319,10 @@ __global__ __launch_bounds__(kAttnThreads, 2) void attn_fwd_bf16_kernel(const At
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  hipLaunchKernelGGL(attn_fwd_bf16_kernel, dim3(grid), dim3(kAttnThreads), 0, stream, a);
+  if (a.block_m == 256)
+    hipLaunchKernelGGL(attn_fwd_bf16_kernel<8>, dim3(grid), dim3(512), 0, stream, a);
+  else
+    hipLaunchKernelGGL(attn_fwd_bf16_kernel<4>, dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 

@@ -22,15 +22,13 @@ struct AttnKernArgs {
   long qs_t, qs_h, ks_t, ks_h, vs_t, vs_h, os_t, os_h;
   int total_q, total_k, k_split;
   int n_ranges, ranges_mode, tiles_per_range;
+  int block_m;  // q rows per workgroup: 128 (4 waves) or 256 (8 waves)
   int Hq, Hkv, G;
   int scale_chunk_tokens;
   unsigned total_wgs, per_xcd;
   float scale_log2;  // softmax_scale * log2(e)
 };
 
-// Q rows one workgroup covers (sizes the grid: tiles_per_range = ceil(max_seqlen_q / kAttnBlockM)).
-constexpr int kAttnBlockM = 128;
-constexpr int kAttnThreads = 256;
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream);
 hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream);

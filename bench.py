@@ -117,6 +117,36 @@ def run_step(inp, ev=None):
     rec("cross", 1)
 
 
+def fp8_leg(inp, core_fl, bf16_tflops, steps):
+    """The same core attention with Q / K / V quantised to e4m3 (per-(chunk, head) absmax scales): kernel-only
+    HIP-event timing, throughput against the fp8 dense peak and against the bf16 kernel, and the deviation from
+    the bf16 kernel's output on the same tensors."""
+    import magi_attn as M
+
+    L, D = inp["L"], inp["D"]
+    cache = inp["cache"]
+    q8, qs = M.quantize_fp8(inp["q"], L)
+    k8, ks = M.quantize_fp8(cache[..., :D], L)
+    v8, vs = M.quantize_fp8(cache[..., D:], L)
+    out8 = torch.empty_like(inp["out"])
+    kw = dict(q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L, out=out8, return_lse=False)
+    M.range_attention(q8, k8, v8, inp["q_ranges"], inp["k_ranges"], L, **kw)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        M.range_attention(q8, k8, v8, inp["q_ranges"], inp["k_ranges"], L, **kw)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    tf = core_fl / (ms * 1e-3) / 1e12
+    a, b = out8[::97].double().flatten(), inp["out"][::97].double().flatten()
+    cos = (torch.dot(a, b) / (a.norm() * b.norm())).item()
+    return {"kernel": "attn_fwd_fp8_kernel", "achieved": round(tf, 2), "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
+            "frac": round(tf / PEAK_FP8_TFLOPS, 4), "ms": round(ms, 3), "speedup_vs_bf16": round(tf / bf16_tflops, 3),
+            "cosine_vs_bf16_output": round(cos, 5), "max_abs_vs_bf16_output": round((a - b).abs().max().item(), 5)}
+
+
 def cpu_baseline(inp, rows_per_chunk=6144):
     """CPU oracle (torch SDPA fp32, one call per range) on a bounded sample of the workload:
     the first rows_per_chunk queries of every denoising chunk, the 6 (= Hq/Hkv) q heads of KV
@@ -205,6 +235,7 @@ def main():
                               "traffic": None, "ms": round(kern_ms["prologue"], 4)},
         "cross_attention_ms": round(kern_ms["cross"], 4),
     }
+    result["fp8"] = fp8_leg(inp, core_fl, core_tflops, args.steps)
     if not args.no_cpu_baseline:
         cb, o_cpu, idx = cpu_baseline(inp)
         got = inp["out"][idx.to(dev), : inp["Hq"] // inp["Hkv"]].float().cpu()

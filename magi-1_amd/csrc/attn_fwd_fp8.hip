@@ -1,6 +1,402 @@
-// fp8-e4m3 range attention forward and the per-(chunk, head) quantiser (placeholder until built).
+// fp8 (OCP e4m3fn) range attention forward and the per-(chunk, head) quantiser, for gfx950.
+//
+// Same organisation as the bf16 kernel (S^T = K Q^T, one query per lane column, online softmax in
+// fp32, O^T = V^T P^T), built on v_mfma_f32_32x32x64_f8f6f4, which runs at twice the bf16 rate:
+//   * K / V tiles are 64 rows x 128 bytes; the transposing LDS read is ds_read_b64_tr_b8;
+//   * P is quantised to e4m3 after scaling by 2^8 (P <= 1 so P * 256 <= 256 < 448), the factor is
+//     folded into the exponent of exp2 and divided out with the row sum;
+//   * Q, K, V carry one fp32 scale per (chunk of `scale_chunk_tokens` tokens, head).  The key axis
+//     is walked in pieces that never cross a scale chunk (nor the boundary between the two key
+//     segments), so inside a tile the K and V scales are wave-uniform scalars: the K scale joins
+//     the softmax scale, the V scale (relative to the largest V scale of the range) joins the exp2
+//     exponent, and the Q scale is a per-lane constant because a lane owns one query.
 #include "kernels.h"
+
 namespace magi {
-hipError_t launch_attn_fwd_fp8(const AttnKernArgs&, hipStream_t) { return hipErrorNotSupported; }
-hipError_t launch_quantize_fp8(const char*, long, long, char*, float*, int, int, int, hipStream_t) { return hipErrorNotSupported; }
+namespace {
+
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+typedef int i32x2 __attribute__((ext_vector_type(2)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+
+#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
+#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
+
+constexpr int BN = 64;
+constexpr int ROW_BYTES = 128;  // D = 128 fp8
+constexpr int TILE_BYTES = BN * ROW_BYTES;
+constexpr int MAX_SORT = 256;
+constexpr int NW = 4;
+constexpr int BM = 32 * NW;
+constexpr int LOADS = 8 / NW;  // direct loads per wave per matrix per tile (8 rows each)
+constexpr float P_SHIFT = 8.f;
+
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
+  f32x2 x = {a, b};
+  bf16x2 r = __builtin_convertvector(x, bf16x2);
+  return __builtin_bit_cast(unsigned, r);
+}
+
+__device__ __forceinline__ void load_range(const int* r, int mode, int i, int total, int& s, int& e) {
+  if (mode == 0) {
+    s = r[2 * i];
+    e = r[2 * i + 1];
+  } else {
+    s = r[i];
+    e = r[i + 1];
+  }
+  s = max(0, min(s, total));
+  e = max(s, min(e, total));
+}
+
+__global__ __launch_bounds__(64 * NW, 2) void attn_fwd_fp8_kernel(const AttnKernArgs a) {
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[2][2][TILE_BYTES];  // [buffer][K|V]
+  __shared__ int s_sel;
+
+  const int tid = threadIdx.x;
+  const unsigned id = blockIdx.x;
+  const unsigned f = (id & 7u) * a.per_xcd + (id >> 3);
+  if (f >= a.total_wgs) return;
+  const unsigned per_range = (unsigned)a.tiles_per_range * (unsigned)a.G;
+  const unsigned per_kvh = (unsigned)a.n_ranges * per_range;
+  const unsigned kvh = f / per_kvh;
+  unsigned rem = f - kvh * per_kvh;
+  const unsigned rslot = rem / per_range;
+  rem -= rslot * per_range;
+  const unsigned tile = rem / (unsigned)a.G;
+  const unsigned hg = rem - tile * (unsigned)a.G;
+  const int h = (int)(kvh * a.G + hg);
+
+  int ridx;
+  if (a.n_ranges <= MAX_SORT) {
+    if (tid < a.n_ranges) {
+      int s, e;
+      load_range(a.k_ranges, a.ranges_mode, tid, a.total_k, s, e);
+      const int my = e - s;
+      int rank = 0;
+      for (int j = 0; j < a.n_ranges; ++j) {
+        int sj, ej;
+        load_range(a.k_ranges, a.ranges_mode, j, a.total_k, sj, ej);
+        const int lj = ej - sj;
+        rank += (lj > my) || (lj == my && j < tid);
+      }
+      if (rank == (int)rslot) s_sel = tid;
+    }
+    __syncthreads();
+    ridx = __builtin_amdgcn_readfirstlane(s_sel);
+  } else {
+    ridx = a.n_ranges - 1 - (int)rslot;
+  }
+  int qs, qe, ks, ke;
+  load_range(a.q_ranges, a.ranges_mode, ridx, a.total_q, qs, qe);
+  load_range(a.k_ranges, a.ranges_mode, ridx, a.total_k, ks, ke);
+  const int q0 = qs + (int)tile * BM;
+  if (q0 >= qe) return;
+
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int l = tid & 63, i = l & 31, g = l >> 5;
+  const int q_row = q0 + 32 * w + i;
+  const bool row_ok = q_row < qe;
+
+  if (ke <= ks) {
+    if (row_ok) {
+      char* op = a.out + (long)q_row * a.os_t + (long)h * a.os_h + g * 128;
+#pragma unroll
+      for (int c = 0; c < 8; ++c) *(u32x4*)(op + c * 16) = u32x4{0, 0, 0, 0};
+      if (a.lse && g == 0) a.lse[(long)h * a.total_q + q_row] = -__builtin_inff();
+    }
+    return;
+  }
+
+  // ---- Q fragments: lane (i, g) holds Q[row i][64kk + 32g .. +32] for kk = 0, 1 ----
+  const int C = a.scale_chunk_tokens;
+  const int qr = min(q_row, qe - 1);
+  i32x8 qf[2];
+  {
+    const char* qp = a.q + (long)qr * a.qs_t + (long)h * a.qs_h + g * 32;
+#pragma unroll
+    for (int kk = 0; kk < 2; ++kk) {
+      const i32x4 lo = *(const i32x4*)(qp + kk * 64);
+      const i32x4 hi = *(const i32x4*)(qp + kk * 64 + 16);
+      qf[kk] = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    }
+  }
+  const float q_sc = a.q_scale[(long)(qr / C) * a.Hq + h];  // this lane's query scale
+
+  // largest V scale of the key range (reference for the relative V scale folded into exp2)
+  float v_max = 0.f;
+  for (int cidx = ks / C; cidx <= (ke - 1) / C; ++cidx) v_max = fmaxf(v_max, a.v_scale[(long)cidx * a.Hkv + kvh]);
+  const float log2_vmax = __builtin_amdgcn_logf(v_max);
+
+  // ---- tile loader: wave w fills rows 8*(w + NW*j) .. +7; lane l sits at row +(l >> 3), slot l & 7 ----
+  const int lrow = l >> 3, slot = l & 7;
+  const int row_in_tile0 = 8 * w + lrow;
+  const int kchunk = slot ^ (4 * (w & 1) + (lrow >> 1));                    // K: chunk ^= (row >> 1) & 7
+  const int vchunk = slot ^ ((((lrow >> 1) & 1) | ((w & 1) << 1)) << 1);    // V: chunk ^= f(row >> 1) << 1
+  const long ks_t = a.ks_t, vs_t = a.vs_t;
+  const int k_split = a.k_split;
+  const long k2_delta = a.k2 ? (a.k2 - a.k) - (long)k_split * ks_t : 0;
+  const long v2_delta = a.v2 ? (a.v2 - a.v) - (long)k_split * vs_t : 0;
+  const char* const kcolp = a.k + (long)kvh * a.ks_h + kchunk * 16;
+  const char* const vcolp = a.v + (long)kvh * a.vs_h + vchunk * 16;
+
+  // The key range is walked in pieces [k0, pe) that stay inside one scale chunk and one key segment.
+  auto piece_end = [&](int k0) {
+    int pe = min(ke, (k0 / C + 1) * C);
+    if (k0 < k_split) pe = min(pe, k_split);
+    return pe;
+  };
+  auto issue_tile = [&](int k0, int pe, int buf) {
+    const bool second = k0 >= k_split;
+    const char* kb = kcolp + (second ? k2_delta : 0);
+    const char* vb = vcolp + (second ? v2_delta : 0);
+#pragma unroll
+    for (int j = 0; j < LOADS; ++j) {
+      const int row = min(k0 + row_in_tile0 + 8 * NW * j, pe - 1);
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kb + (long)row * ks_t), LDS_PTR(void, &smem[buf][0][(w + j * NW) * 1024]),
+                                       16, 0, 0);
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vb + (long)row * vs_t), LDS_PTR(void, &smem[buf][1][(w + j * NW) * 1024]),
+                                       16, 0, 0);
+    }
+  };
+
+  // ---- per-lane LDS read bases ----
+  // K (A operand): row 32t + i, chunks 4kk + 2g + u  ->  (base_k ^ (u << 4) ^ (kk << 6)) + t * 4096
+  const int base_k = i * ROW_BYTES + (((((i >> 1) & 7) ^ (2 * g))) << 4);
+  // V^T via ds_read_b64_tr_b8: in a 16-lane group lane pair (2r', 2r'+1) supplies row r' of 8, lane gets d column l & 15.
+  // Operand slot e = 16t + 4b + r holds key 32t + 8b + 4g + r; read n2 covers t = n2 >> 1, b in {2(n2&1), +1}.
+  const int lam = l & 15, rp = lam >> 1, dblk = (l >> 4) & 1;
+  const int rho0 = 4 * g + (rp & 3) + 8 * (rp >> 2);
+  const int f_v = (lam >> 2) & 3;
+  const int base_v = rho0 * ROW_BYTES + (((2 * f_v) | dblk) << 4) + (l & 1) * 8;
+
+  f32x16 o_acc[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int v = 0; v < 16; ++v) o_acc[mb][v] = 0.f;
+  float m_run = -__builtin_inff();  // running max in scaled log2 units
+  float l_run = 0.f;
+  const bool wave_on = (q0 + 32 * w) < qe;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const float c_q = a.scale_log2 * q_sc;  // softmax scale * log2(e) * q scale
+
+  int k0 = ks, pe = piece_end(ks);
+  issue_tile(k0, pe, 0);
+  int buf = 0;
+  while (k0 < ke) {
+    int k1 = k0 + BN, pe1 = pe;  // the tile after this one
+    if (k1 >= pe) {
+      k1 = pe;
+      pe1 = (k1 < ke) ? piece_end(k1) : ke;
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (k1 < ke) issue_tile(k1, pe1, buf ^ 1);
+    if (wave_on) {
+      const unsigned char* Kt = &smem[buf][0][0];
+      const unsigned char* Vt = &smem[buf][1][0];
+      const int cidx = k0 / C;
+      const float k_sc = a.k_scale[(long)cidx * a.Hkv + kvh];
+      const float v_sc = a.v_scale[(long)cidx * a.Hkv + kvh];
+      const float c = c_q * k_sc;                                             // per-lane score scale of this tile
+      const float shift = P_SHIFT + __builtin_amdgcn_logf(v_sc) - log2_vmax;  // <= 8
+      const float unshift = __builtin_amdgcn_exp2f(-shift);
+
+      auto read_k = [&](int t, int kk) -> i32x8 {
+        const int o = (base_k ^ (kk << 6)) + t * 4096;
+        const i32x4 lo = *LDS_PTR(const i32x4, Kt + o);
+        const i32x4 hi = *LDS_PTR(const i32x4, Kt + (o ^ 16));
+        return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      };
+      auto read_v = [&](int mb) -> i32x8 {
+        const int o = base_v ^ (mb << 5);
+        i32x2 r[4];
+#pragma unroll
+        for (int n2 = 0; n2 < 4; ++n2)
+          r[n2] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(i32x2, Vt + (o + (n2 >> 1) * 4096 + (n2 & 1) * 2048)));
+        return i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
+      };
+
+      i32x8 ka[4], va[4];
+#pragma unroll
+      for (int n = 0; n < 4; ++n) ka[n] = read_k(n >> 1, n & 1);
+      f32x16 s_acc[2];
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[2 * t], qf[0], zero16, 0, 0, 0, 0, 0, 0);
+        s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[2 * t + 1], qf[1], s_acc[t], 0, 0, 0, 0, 0, 0);
+        va[2 * t] = read_v(2 * t);
+        va[2 * t + 1] = read_v(2 * t + 1);
+      }
+      if (k0 + BN > pe) {  // ragged last tile of a piece
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = k0 + 32 * t + 8 * (v >> 2) + 4 * g + (v & 3);
+            if (key >= pe) s_acc[t][v] = -__builtin_inff();
+          }
+      }
+      float mx = s_acc[0][0];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[t][v]);
+      mx = fmaxf(mx, __shfl_xor(mx, 32));
+      const float m_new = fmaxf(m_run, mx * c);
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      const float mc = m_new - shift;
+      m_run = m_new;
+      float psum = 0.f;
+      i32x8 pb;
+#pragma unroll
+      for (int n = 0; n < 8; ++n) {  // dword n = slots 4n .. 4n+3 = s_acc[n >> 2][4 (n & 3) .. +3]
+        const float p0 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 0] * c - mc);
+        const float p1 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 1] * c - mc);
+        const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2] * c - mc);
+        const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3] * c - mc);
+        psum += (p0 + p1) + (p2 + p3);
+        int u = 0;
+        u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
+        u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
+        pb[n] = u;
+      }
+      l_run = l_run * alpha + psum * unshift;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+      }
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+        o_acc[mb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va[mb], pb, o_acc[mb], 0, 0, 0, 0, 0, 0);
+    }
+    k0 = k1;
+    pe = pe1;
+    buf ^= 1;
+  }
+
+  if (!wave_on) return;
+  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float inv = v_max * __builtin_amdgcn_exp2f(-P_SHIFT) / l_tot;
+  if (row_ok) {
+    char* op = a.out + (long)q_row * a.os_t + (long)h * a.os_h;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int b = 0; b < 4; ++b) {
+        const int d = 32 * mb + 8 * b + 4 * g;
+        u32x2 pk;
+        pk[0] = pack_bf16x2(o_acc[mb][4 * b + 0] * inv, o_acc[mb][4 * b + 1] * inv);
+        pk[1] = pack_bf16x2(o_acc[mb][4 * b + 2] * inv, o_acc[mb][4 * b + 3] * inv);
+        *(u32x2*)(op + d * 2) = pk;
+      }
+    if (a.lse && g == 0)
+      a.lse[(long)h * a.total_q + q_row] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Quantiser: absmax per (chunk, head) -> scale = max(absmax, tiny) / 448; y = e4m3(clamp(x / scale)).
+// ------------------------------------------------------------------------------------------------
+constexpr int QT = 256;
+
+__global__ __launch_bounds__(QT) void fill_zero_kernel(unsigned* p, int n) {
+  const int i = blockIdx.x * QT + threadIdx.x;
+  if (i < n) p[i] = 0u;
+}
+
+// grid (slices, H, n_chunks); 16 lanes x 16 bytes per (token, head) row; result: max |x| bits in amax[c*H + h]
+__global__ __launch_bounds__(QT) void absmax_kernel(const char* x, long xs_t, long xs_h, unsigned* amax, int T, int H,
+                                                    int chunk_tokens) {
+  __shared__ unsigned s_red[QT / 64];
+  const int c = blockIdx.z, h = blockIdx.y;
+  const int t_begin = c * chunk_tokens, t_end = min(T, t_begin + chunk_tokens);
+  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
+  unsigned m = 0u;
+  for (int t = t_begin + blockIdx.x * (QT / 16) + sub; t < t_end; t += gridDim.x * (QT / 16)) {
+    const u32x4 v = *(const u32x4*)(x + (long)t * xs_t + (long)h * xs_h + lane16 * 16);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      m = max(m, (v[j] << 16) & 0x7fffffffu);
+      m = max(m, v[j] & 0x7fff0000u);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o));
+  if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+#pragma unroll
+    for (int j = 1; j < QT / 64; ++j) m = max(m, s_red[j]);
+    atomicMax(&amax[c * H + h], m);  // non-negative floats order like their bit patterns
+  }
+}
+
+__global__ __launch_bounds__(QT) void finalize_scales_kernel(float* scales, int n) {
+  const int i = blockIdx.x * QT + threadIdx.x;
+  if (i < n) scales[i] = fmaxf(scales[i] / 448.f, 1e-12f);
+}
+
+// one thread per 8 elements
+__global__ __launch_bounds__(QT) void quantize_kernel(const char* x, long xs_t, long xs_h, char* y, const float* scales,
+                                                      int T, int H, int chunk_tokens) {
+  const long gid = (long)blockIdx.x * QT + threadIdx.x;
+  const long row = gid >> 4;
+  const int part = (int)(gid & 15);
+  if (row >= (long)T * H) return;
+  const int t = (int)(row / H), h = (int)(row % H);
+  const float sc = scales[(long)(t / chunk_tokens) * H + h];
+  const u32x4 v = *(const u32x4*)(x + (long)t * xs_t + (long)h * xs_h + part * 16);
+  float fv[8];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    fv[2 * j] = __builtin_bit_cast(float, v[j] << 16);
+    fv[2 * j + 1] = __builtin_bit_cast(float, v[j] & 0xffff0000u);
+  }
+#pragma unroll
+  for (int j = 0; j < 8; ++j) fv[j] = fminf(fmaxf(fv[j] / sc, -448.f), 448.f);
+  u32x2 o;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    int u = 0;
+    u = __builtin_amdgcn_cvt_pk_fp8_f32(fv[4 * j], fv[4 * j + 1], u, false);
+    u = __builtin_amdgcn_cvt_pk_fp8_f32(fv[4 * j + 2], fv[4 * j + 3], u, true);
+    o[j] = (unsigned)u;
+  }
+  *(u32x2*)(y + row * 128 + part * 8) = o;
+}
+
+}  // namespace
+
+hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream) {
+  const unsigned grid = a.per_xcd * 8u;
+  hipLaunchKernelGGL(attn_fwd_fp8_kernel, dim3(grid), dim3(64 * NW), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
+                               int chunk_tokens, hipStream_t stream) {
+  const int n_chunks = (T + chunk_tokens - 1) / chunk_tokens;
+  const int n = n_chunks * H;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((n + QT - 1) / QT), dim3(QT), 0, stream, (unsigned*)scales, n);
+  const int rows_per_pass = QT / 16;
+  int slices = (min(chunk_tokens, T) + rows_per_pass * 8 - 1) / (rows_per_pass * 8);
+  slices = max(1, min(slices, 256));
+  hipLaunchKernelGGL(absmax_kernel, dim3(slices, H, n_chunks), dim3(QT), 0, stream, x, x_stride_t, x_stride_h,
+                     (unsigned*)scales, T, H, chunk_tokens);
+  hipLaunchKernelGGL(finalize_scales_kernel, dim3((n + QT - 1) / QT), dim3(QT), 0, stream, scales, n);
+  const long threads = (long)T * H * 16;
+  hipLaunchKernelGGL(quantize_kernel, dim3((unsigned)((threads + QT - 1) / QT)), dim3(QT), 0, stream, x, x_stride_t,
+                     x_stride_h, y, scales, T, H, chunk_tokens);
+  return hipGetLastError();
+}
+
 }  // namespace magi

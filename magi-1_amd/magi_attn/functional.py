@@ -252,3 +252,19 @@ def head_norm(x: torch.Tensor, gamma, beta, eps: float = 1e-6, norm_kind: int = 
         L.check(L.lib().magi_head_norm(x.data_ptr(), x.stride(0), x.stride(1), _ptr(g), _ptr(b), y.data_ptr(), S, H, D,
                                        int(norm_kind), float(eps), _stream()))
     return y
+
+
+def quantize_fp8(x: torch.Tensor, chunk_tokens: int):
+    """x [T, H, 128] bf16 (strided heads allowed) -> (y [T, H, 128] float8_e4m3fn, scales [ceil(T/chunk), H] fp32)
+    with x ~= y * scales[t // chunk_tokens, h]: per-(chunk, head) absmax / 448, saturating OCP e4m3fn."""
+    _check_thd(x, "x")
+    if x.dtype != torch.bfloat16:
+        raise TypeError("x must be bf16")
+    T, H, D = x.shape
+    n_chunks = (T + chunk_tokens - 1) // chunk_tokens
+    y = torch.empty((T, H, D), dtype=torch.float8_e4m3fn, device=x.device)
+    scales = torch.empty((n_chunks, H), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        L.check(L.lib().magi_quantize_fp8(x.data_ptr(), x.stride(0), x.stride(1), y.data_ptr(), scales.data_ptr(), T, H, D,
+                                          int(chunk_tokens), _stream()))
+    return y, scales

@@ -1,0 +1,125 @@
+"""GPU tests of the fp8-e4m3 path: quantiser (bit-exact against the oracle's quantiser) and the fp8
+attention kernel against the fp32 oracle.
+
+The reference has no fp8 attention, so this path's parity is unpinned by the reference; it is
+pinned here by (a) the quantiser's bit-exact agreement with the oracle's saturating e4m3fn
+quantiser, (b) the fp32 oracle evaluated on the ORIGINAL bf16 inputs with the tolerance below, and
+(c) the fp32 oracle evaluated on the DEQUANTISED inputs, which isolates the kernel's own error
+(P quantisation + MFMA accumulation) from the input quantisation error.
+
+Stated tolerance, per head, against the fp32 oracle on the original inputs (N(0,1) values, per-head
+normalised Q / K): cosine >= 0.998 and max-abs <= 2^-5 * max|V| (an output row is a convex combination
+of V rows, e4m3 rounds a value v to within 2^-4 |v|; half of that bound, which also has to absorb the
+score errors, holds on every seeded case here; at benchmark sizes the averaging over ~10^5 keys brings
+max-abs below 1e-2).  Against the dequantised-input oracle: max-abs <= 4e-2 and cosine >= 0.9995."""
+import numpy as np
+import pytest
+import torch
+
+import magi_attn as M
+from oracle import magi_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _per_head(out, ref):
+    o = out.double().cpu()
+    r = ref.double().cpu()
+    err = (o - r).abs().amax(dim=(0, 2))
+    cos = (o * r).sum(dim=(0, 2)) / (o.pow(2).sum(dim=(0, 2)).sqrt() * r.pow(2).sum(dim=(0, 2)).sqrt()).clamp_min(1e-30)
+    return err.max().item(), cos.min().item()
+
+
+def test_quantiser_bit_exact_with_oracle(dev):
+    g = torch.Generator().manual_seed(0)
+    x = (torch.randn(333, 6, 128, generator=g) * torch.tensor([0.1, 1, 30, 1, 2, 1e-3])[None, :, None]).bfloat16()
+    x[5, 0] = 0  # a zero row
+    y, sc = M.quantize_fp8(x.to(dev), 100)
+    y_ref, sc_ref = O.quantize_per_head_chunk(x, 100)
+    assert sc.shape == (4, 6) and torch.equal(sc.cpu(), sc_ref)
+    assert torch.equal(y.cpu().view(torch.uint8), y_ref.view(torch.uint8))
+    assert y.float().abs().max() == 448  # absmax lands on the top code, nothing becomes NaN
+    # strided input (the K half of an interleaved cache) and an all-zero tensor
+    kv = torch.randn(64, 2, 256, generator=g).bfloat16()
+    y2, s2 = M.quantize_fp8(kv.to(dev)[..., :128], 64)
+    y2r, s2r = O.quantize_per_head_chunk(kv[..., :128], 64)
+    assert torch.equal(y2.cpu().view(torch.uint8), y2r.view(torch.uint8)) and torch.equal(s2.cpu(), s2r)
+    z, sz = M.quantize_fp8(torch.zeros(10, 1, 128, dtype=torch.bfloat16, device=dev), 10)
+    assert torch.all(z.float() == 0) and torch.all(sz > 0)
+
+
+@pytest.mark.parametrize("L,dn,sp,Hq,Hkv,C", [(128, 1, 0, 1, 1, 128), (64, 2, 0, 2, 1, 64), (200, 3, 1, 6, 2, 200),
+                                              (77, 2, 2, 3, 1, 50), (300, 2, 1, 6, 1, 1000), (1536, 3, 0, 24, 8, 1536)])
+def test_fp8_attention_parity(dev, L, dn, sp, Hq, Hkv, C):
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=4234 + L)
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    q8, qs = M.quantize_fp8(q.to(dev), C)
+    k8, ks = M.quantize_fp8(k.to(dev), C)
+    v8, vs = M.quantize_fp8(v.to(dev), C)
+    tq = torch.tensor(qr, device=dev)
+    tk = torch.tensor(kr, device=dev)
+    out, lse = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=C)
+    assert out.dtype == torch.bfloat16 and torch.isfinite(out).all()
+    err, cos = _per_head(out, O.range_attention(q, k, v, qr, kr))
+    assert err <= 2 ** -5 * v.float().abs().max().item() and cos >= 0.998, (err, cos)
+    deq = O.fp8_range_attention(q8.cpu(), k8.cpu(), v8.cpu(), qs.cpu(), ks.cpu(), vs.cpu(), C, qr, kr)
+    err, cos = _per_head(out, deq)
+    assert err <= 4e-2 and cos >= 0.9995, (err, cos)
+    lse_ref = O.range_attention_lse(O.dequantize_per_head_chunk(q8.cpu(), qs.cpu(), C),
+                                    O.dequantize_per_head_chunk(k8.cpu(), ks.cpu(), C), v, qr, kr)
+    assert (lse.cpu() - lse_ref).abs().max() < 1e-3
+
+
+def test_fp8_uneven_scales_and_two_segments(dev):
+    """Chunks with very different magnitudes (the per-chunk scales must be honoured, including the
+    relative V scale folded into the exponent) and a key axis split over two buffers."""
+    L, sp, dn, Hq, Hkv = 96, 2, 2, 4, 2
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=77)
+    mag = torch.tensor([1.0, 8.0, 0.25, 3.0]).repeat_interleave(L)[:, None, None]
+    v = (v.float() * mag).bfloat16()
+    k = (k.float() * mag.flip(0) ** 0.25).bfloat16()
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    q8, qs = M.quantize_fp8(q.to(dev), L)
+    k8, ks = M.quantize_fp8(k.to(dev), L)
+    v8, vs = M.quantize_fp8(v.to(dev), L)
+    tq, tk = torch.tensor(qr, device=dev), torch.tensor(kr, device=dev)
+    kw = dict(q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L)
+    out, _ = M.range_attention(q8, k8, v8, tq, tk, L, **kw)
+    deq = O.fp8_range_attention(q8.cpu(), k8.cpu(), v8.cpu(), qs.cpu(), ks.cpu(), vs.cpu(), L, qr, kr)
+    o = out.double().cpu()
+    assert ((o - deq.double()).abs().max() / deq.abs().max()).item() <= 4e-2
+    split = sp * L + 40
+    out2, _ = M.range_attention(q8, k8[:split], v8[:split], tq, tk, L, k2=k8[split:].clone(), v2=v8[split:].clone(),
+                                k_split=split, **kw)
+    # the split moves tile boundaries (a piece ends at the split), so rounding may differ by a bf16 ulp or two
+    assert (out2.float() - out.float()).abs().max().item() <= 4e-2 * deq.abs().max().item()
+
+
+def test_fp8_full_size_720p_speedup_and_accuracy(dev):
+    """Benchmark shape in fp8: sampled-row accuracy against fp32 math on the original tensors."""
+    L, dn, sp, Hq, Hkv, D = 21600, 4, 8, 48, 8, 128
+    g = torch.Generator(device=dev).manual_seed(5234)
+    q = torch.randn(dn * L, Hq, D, device=dev, generator=g)
+    q = (q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    k = torch.randn((sp + dn) * L, Hkv, D, device=dev, generator=g)
+    k = (k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
+    v = torch.randn((sp + dn) * L, Hkv, D, device=dev, generator=g).bfloat16()
+    q8, qs = M.quantize_fp8(q, L)
+    k8, ks = M.quantize_fp8(k, L)
+    v8, vs = M.quantize_fp8(v, L)
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    tq, tk = torch.tensor(qr, device=dev), torch.tensor(kr, device=dev)
+    out, _ = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L,
+                               return_lse=False)
+    torch.cuda.synchronize()
+    G = Hq // Hkv
+    rs = np.random.default_rng(0)
+    for i in range(dn):
+        rows = torch.tensor(np.sort(rs.choice(L, 64, replace=False)) + i * L, device=dev)
+        ke = int(kr[i, 1])
+        ref = torch.empty(64, Hq, D, device=dev)
+        for hk in range(Hkv):
+            s = torch.einsum("rgd,kd->rgk", q[rows, hk * G:(hk + 1) * G].float(), k[:ke, hk].float()) * D ** -0.5
+            ref[:, hk * G:(hk + 1) * G] = torch.einsum("rgk,kd->rgd", torch.softmax(s, -1), v[:ke, hk].float())
+        err, cos = _per_head(out[rows], ref)
+        assert err <= 1e-2 and cos >= 0.998, (i, err, cos)

@@ -179,6 +179,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="720p-24B", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-fp8", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="run one plain device copy of known size (for scaling FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
@@ -235,7 +238,12 @@ def main():
                               "traffic": None, "ms": round(kern_ms["prologue"], 4)},
         "cross_attention_ms": round(kern_ms["cross"], 4),
     }
-    result["fp8"] = fp8_leg(inp, core_fl, core_tflops, args.steps)
+    if not args.no_fp8:
+        result["fp8"] = fp8_leg(inp, core_fl, core_tflops, args.steps)
+    if args.copy_calibration:
+        inp["xout"].copy_(inp["out"])  # reads and writes out.numel() * 2 bytes each
+        torch.cuda.synchronize()
+        result["copy_calibration_bytes_each_way"] = inp["out"].numel() * 2
     if not args.no_cpu_baseline:
         cb, o_cpu, idx = cpu_baseline(inp)
         got = inp["out"][idx.to(dev), : inp["Hq"] // inp["Hkv"]].float().cpu()

@@ -27,6 +27,9 @@ import torch
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
+# HBM-side bytes per launch on the 720p workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
+# plain copy of known size in the same run (FETCH_SIZE x2.0, WRITE_SIZE x1.0): profiles/bench_720p_hbm_traffic_pmc.txt
+MEASURED_TRAFFIC = {"720p-24B": {"core": 88.6e9 + 1.09e9, "prologue": 1.451e9 + 1.478e9, "fp8": 33.3e9 + 1.11e9}}
 
 WORKLOADS = {
     # name: (T_lat frames per chunk, H, W, denoise chunks, prefix chunks, Hq, Hkv)
@@ -232,10 +235,11 @@ def main():
                    "core_flops": core_fl, "cross_flops": cross_fl},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_kernel", "achieved": round(core_tflops, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(core_tflops / PEAK_BF16_TFLOPS, 4),
-                     "traffic": None, "ms": round(kern_ms["core"], 3)},
+                     "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("core"), "ms": round(kern_ms["core"], 3)},
         "roofline_prologue": {"bound": "hbm", "kernel": "prologue_kernel", "achieved": round(pro_gbs, 1),
                               "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(pro_gbs / PEAK_HBM_GBS, 4),
-                              "traffic": None, "ms": round(kern_ms["prologue"], 4)},
+                              "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("prologue"),
+                              "ms": round(kern_ms["prologue"], 4)},
         "cross_attention_ms": round(kern_ms["cross"], 4),
     }
     if not args.no_fp8:

@@ -105,6 +105,7 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   if (const char* e = std::getenv("MAGI_ATTN_BLOCK_M")) {  // tuning knob: 128 or 256
     if (std::atoi(e) == 256) a.block_m = 256;
   }
+  if (const char* e = std::getenv("MAGI_ATTN_VARIANT")) a.variant = std::atoi(e);  // tuning knob
   a.tiles_per_range = (p->max_seqlen_q + a.block_m - 1) / a.block_m;
   a.Hq = p->Hq;
   a.Hkv = p->Hkv;

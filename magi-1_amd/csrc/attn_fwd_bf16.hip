@@ -1,8 +1,8 @@
 // Range attention forward, bf16 in / bf16 out, fp32 online softmax, for gfx950 (MI355X).
 //
 // One workgroup = NW wavefronts = 32*NW query rows of one (range, q head); wave w owns rows
-// 32w..32w+31.  Key/value rows stream through LDS in tiles of 64, double buffered, filled by
-// direct global->LDS loads (no register staging).
+// 32w..32w+31.  Key/value rows stream through LDS in tiles of BN keys held in a ring of NSTAGE
+// stages, filled by direct global->LDS loads (no register staging) issued NSTAGE-1 tiles ahead.
 //
 // The scores are computed transposed, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: the
 // accumulator layout then puts ONE query per lane column (lane % 32) and spreads the keys over
@@ -11,11 +11,17 @@
 // product O^T = V^T P^T.  V^T is fetched from the row-major V tile with the transposing LDS
 // read ds_read_b64_tr_b16.
 //
-// LDS tile layout: 64 rows of 256 bytes; the 16-byte chunk c of row r lives at chunk
+// LDS tile layout: rows of 256 bytes; the 16-byte chunk c of row r lives at chunk
 // c ^ (r & 15) for K (conflict-free ds_read_b128 down a column of rows) and at
 // c ^ ((r & 3) << 2) for V (conflict-free transposing reads of 4-row groups).  A direct load
 // places lane l's 16 bytes at base + 16*l, so the swizzle is applied on the global side: lane
 // l fetches the logical chunk that belongs at its fixed LDS slot.
+//
+// A single wavefront cannot keep the MFMA pipe busy (in-order issue, ~5 cycles between its VALU
+// instructions, LDS and MFMA latencies in series): throughput comes from several waves per SIMD
+// in different phases.  The kernel is therefore instantiated for 2 waves / SIMD (BN = 64, deep
+// operand prefetch, <= 256 VGPRs) and for 3 waves / SIMD (BN = 32, shallow prefetch, <= 168
+// VGPRs, 48 KB of LDS per workgroup).
 //
 // Work decomposition: blockIdx -> (kv head, range slot, q tile, q head within the GQA group),
 // laid out so that the workgroups an XCD receives (blockIdx % 8) share a KV head and walk the
@@ -38,9 +44,7 @@ typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 #define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
 #define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
-constexpr int BN = 64;          // keys per tile
 constexpr int ROW_BYTES = 256;  // D = 128 bf16
-constexpr int TILE_BYTES = BN * ROW_BYTES;
 constexpr int MAX_SORT = 256;
 
 __device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
@@ -61,11 +65,25 @@ __device__ __forceinline__ void load_range(const int* r, int mode, int i, int to
   e = max(s, min(e, total));
 }
 
-template <int NW>
-__global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
+// s_waitcnt vmcnt(N), leaving the other counters alone
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+  asm volatile("" ::: "memory");
+}
+
+template <int NW, int BN, int NSTAGE, int OCC>
+__global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
   constexpr int BM = 32 * NW;
-  constexpr int LOADS = 16 / NW;  // direct loads per wave per matrix per tile (4 rows each)
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[2][2][TILE_BYTES];  // [buffer][K|V]
+  constexpr int TILE_BYTES = BN * ROW_BYTES;
+  constexpr int LOADS = BN / (4 * NW);     // direct loads per wave per matrix per tile (4 rows each)
+  constexpr int TILE_LOADS = 2 * LOADS;    // ... per wave per tile
+  constexpr int NT = BN / 32;              // 32-key score tiles per key tile
+  constexpr int NS = BN / 16;              // 16-key slabs per key tile
+  constexpr int DK = OCC >= 3 ? 4 : 8;     // K operands in flight
+  constexpr int DV = OCC >= 3 ? 4 : 8;     // V operands in flight
+  static_assert(LOADS >= 1 && NSTAGE >= 2 && NSTAGE <= 4, "bad tile configuration");
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[NSTAGE][2][TILE_BYTES];  // [stage][K|V]
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -136,9 +154,9 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKer
 
   // ---- K/V tile loader: wave w fills rows 4*(w + NW*j) .. +3; lane l sits at row +(l >> 4), slot l & 15 ----
   const int lrow = l >> 4, slot = l & 15;
-  const int row_in_tile0 = 4 * w + lrow;                    // + 4*NW*j
-  const int kchunk = slot ^ ((4 * (w & 3) + lrow) & 15);    // logical chunk that belongs in this K slot
-  const int vchunk = slot ^ (lrow << 2);                    // ... in this V slot
+  const int row_in_tile0 = 4 * w + lrow;                  // + 4*NW*j
+  const int kchunk = slot ^ ((4 * (w & 3) + lrow) & 15);  // logical chunk that belongs in this K slot
+  const int vchunk = slot ^ (lrow << 2);                  // ... in this V slot
   const long ks_t = a.ks_t, vs_t = a.vs_t;
   const int k_split = a.k_split;
   const long k2_delta = a.k2 ? (a.k2 - a.k) - (long)k_split * ks_t : 0;
@@ -149,11 +167,12 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKer
   const unsigned vvoff = (unsigned)row_in_tile0 * (unsigned)vs_t + (unsigned)(vchunk * 16);
   const bool small_strides = ks_t * (BN + 4) < (1l << 31) && vs_t * (BN + 4) < (1l << 31);
 
-  auto issue_tile = [&](int k0, int buf) {
-    unsigned char* kdst = &smem[buf][0][w * 1024];
-    unsigned char* vdst = &smem[buf][1][w * 1024];
+  // Always TILE_LOADS load instructions per wave, so outstanding loads can be counted in tiles.
+  auto issue_tile = [&](int k0, int stage) {
+    unsigned char* kdst = &smem[stage][0][w * 1024];
+    unsigned char* vdst = &smem[stage][1][w * 1024];
     const bool interior = small_strides && (k0 + BN <= ke) && (k0 + BN <= k_split || k0 >= k_split);
-    if (interior) {  // uniform base + per-lane 32-bit offset
+    if (interior) {  // wave-uniform base + per-lane 32-bit offset
       const bool second = k0 >= k_split;
       const char* kb = kcolp + (long)k0 * ks_t + (second ? k2_delta : 0);
       const char* vb = vcolp + (long)k0 * vs_t + (second ? v2_delta : 0);
@@ -197,23 +216,37 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKer
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   const int n_tiles = (ke - ks + BN - 1) / BN;
-  issue_tile(ks, 0);
+#pragma unroll
+  for (int p = 0; p < NSTAGE - 1; ++p)
+    if (p < n_tiles) issue_tile(ks + p * BN, p);
+  int stage = 0;
   for (int it = 0; it < n_tiles; ++it) {
-    const int buf = it & 1;
     const int k0 = ks + it * BN;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's share of tile `it` is in LDS
-    __syncthreads();                                   // ... and everybody else's; buffer buf^1 is free
-    if (it + 1 < n_tiles) issue_tile(k0 + BN, buf ^ 1);
+    // tile `it` must have landed; up to NSTAGE-2 younger tiles may still be in flight
+    const int younger = min(NSTAGE - 2, n_tiles - 1 - it);
+    if (NSTAGE >= 4 && younger == 2)
+      wait_vmcnt<2 * TILE_LOADS>();
+    else if (NSTAGE >= 3 && younger == 1)
+      wait_vmcnt<TILE_LOADS>();
+    else
+      wait_vmcnt<0>();
+    __syncthreads();  // everybody's share landed; the stage read in the previous iteration is free again
+    if (it + NSTAGE - 1 < n_tiles) {
+      int st = stage + NSTAGE - 1;
+      if (st >= NSTAGE) st -= NSTAGE;
+      issue_tile(k0 + (NSTAGE - 1) * BN, st);
+    }
+    const unsigned char* Kt = &smem[stage][0][0];
+    const unsigned char* Vt = &smem[stage][1][0];
+    stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
     if (!wave_on) continue;
 
-    const unsigned char* Kt = &smem[buf][0][0];
-    const unsigned char* Vt = &smem[buf][1][0];
-
     // LDS operand fetchers
-    auto read_k = [&](int t, int kk) -> bf16x8 {
-      return *LDS_PTR(const bf16x8, Kt + ((base_k ^ (kk << 5)) + t * 32 * ROW_BYTES));
+    auto read_k = [&](int idx) -> bf16x8 {  // idx = 8t + kk
+      return *LDS_PTR(const bf16x8, Kt + ((base_k ^ ((idx & 7) << 5)) + (idx >> 3) * 32 * ROW_BYTES));
     };
-    auto read_v = [&](int mb, int s) -> bf16x8 {
+    auto read_v = [&](int p) -> bf16x8 {  // p = mb * NS + slab
+      const int mb = p / NS, s = p % NS;
       const int bv = base_v ^ (mb << 6);
       const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * s) * ROW_BYTES)));
       const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * s + 8) * ROW_BYTES)));
@@ -221,28 +254,29 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKer
       return __builtin_bit_cast(bf16x8, va);
     };
 
-    // S^T[key][q] for 64 keys x 32 queries.  Operand reads run one half-tile ahead of the MFMAs
-    // that consume them, and the first V operands are fetched under the second half's MFMAs.
-    f32x16 s_acc[2];
-    bf16x8 ka[8], kb[8], vbuf[8];
+    // S^T[key][q] for BN keys x 32 queries.  K operands run DK reads ahead of the MFMAs that consume
+    // them; the first DV V operands are fetched under the last MFMAs.
+    constexpr int RK = NT * 8;
+    constexpr int RV = NS * 4;
+    f32x16 s_acc[NT];
+    bf16x8 kbuf[DK], vbuf[DV];
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) ka[kk] = read_k(0, kk);
+    for (int idx = 0; idx < DK; ++idx) kbuf[idx] = read_k(idx);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-      s_acc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ka[kk], qf[kk], kk == 0 ? zero16 : s_acc[0], 0, 0, 0);
-      kb[kk] = read_k(1, kk);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-      s_acc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kb[kk], qf[kk], kk == 0 ? zero16 : s_acc[1], 0, 0, 0);
-      vbuf[kk] = read_v(kk >> 2, kk & 3);
+    for (int idx = 0; idx < RK; ++idx) {
+      const int t = idx >> 3, kk = idx & 7;
+      s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kbuf[idx % DK], qf[kk], kk == 0 ? zero16 : s_acc[t], 0, 0, 0);
+      if (idx + DK < RK)
+        kbuf[idx % DK] = read_k(idx + DK);
+      else if (idx + DK - RK < DV)
+        vbuf[idx + DK - RK] = read_v(idx + DK - RK);
+      if (DK == 8 && NT == 2 && idx == 7) __builtin_amdgcn_sched_barrier(0);
     }
     __builtin_amdgcn_sched_barrier(0);
     if (k0 + BN > ke) {  // ragged last tile: keys >= ke do not exist
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < NT; ++t)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
           const int key = k0 + 32 * t + 8 * (v >> 2) + 4 * g + (v & 3);
@@ -252,7 +286,7 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKer
     // online softmax: every value this lane holds belongs to query i
     float mx = s_acc[0][0];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < NT; ++t)
 #pragma unroll
       for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[t][v]);
     mx = fmaxf(mx, __shfl_xor(mx, 32));
@@ -261,9 +295,9 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKer
     const float mc = m_new * c;
     m_run = m_new;
     float psum = 0.f;
-    bf16x8 pb[4];
+    bf16x8 pb[NS];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < NS; ++s) {
       u32x4 pk;
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
@@ -282,15 +316,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKer
         for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
     }
 
-    // O^T[d][q] += V^T[d][key] P^T[key][q]; V operands of d-block mb + 2 are fetched while block mb multiplies
+    // O^T[d][q] += V^T[d][key] P^T[key][q]; V operands run DV reads ahead
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        o_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vbuf[(mb & 1) * 4 + s], pb[s], o_acc[mb], 0, 0, 0);
-        if (mb + 2 < 4) vbuf[(mb & 1) * 4 + s] = read_v(mb + 2, s);
-      }
+    for (int p = 0; p < RV; ++p) {
+      const int mb = p / NS, s = p % NS;
+      o_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vbuf[p % DV], pb[s], o_acc[mb], 0, 0, 0);
+      if (p + DV < RV) vbuf[p % DV] = read_v(p + DV);
     }
   }
 
@@ -320,9 +352,11 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_bf16_kernel(const AttnKer
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
   if (a.block_m == 256)
-    hipLaunchKernelGGL(attn_fwd_bf16_kernel<8>, dim3(grid), dim3(512), 0, stream, a);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2>), dim3(grid), dim3(512), 0, stream, a);
+  else if (a.variant == 1)
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 32, 3, 3>), dim3(grid), dim3(256), 0, stream, a);
   else
-    hipLaunchKernelGGL(attn_fwd_bf16_kernel<4>, dim3(grid), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 

@@ -51,7 +51,8 @@ def test_chunk_causal_parity(dev, L, dn, sp, Hq, Hkv):
     out, lse = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, int(kr.max() - kr.min()))
     assert out.dtype == torch.bfloat16 and out.shape == q.shape and lse.shape == (Hq, dn * L)
     _cmp(out, ref, f"L={L}")
-    assert (lse.cpu() - lse_ref).abs().max() < 2e-3
+    # Q is pre-multiplied by scale * log2(e) and re-rounded to bf16 once per workgroup: ~1e-3 on the logits
+    assert (lse.cpu() - lse_ref).abs().max() < 5e-3
 
 
 def test_sliding_window_ranges_and_unsorted_order(dev):

@@ -20,7 +20,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 constexpr int D = 128;
 constexpr int THREADS = 256;
 constexpr int GROUPS = THREADS / 8;  // rows in flight per workgroup
-constexpr int TOK_PER_BLOCK = 4;
+constexpr int TOK_PER_BLOCK = 1;
 
 __device__ __forceinline__ void unpack8(const u32x4 v, float* f) {
 #pragma unroll

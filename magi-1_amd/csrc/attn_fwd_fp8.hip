@@ -54,7 +54,7 @@ __device__ __forceinline__ void load_range(const int* r, int mode, int i, int to
   e = max(s, min(e, total));
 }
 
-__global__ __launch_bounds__(64 * NW, 2) void attn_fwd_fp8_kernel(const AttnKernArgs a) {
+__global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKernArgs a) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[2][2][TILE_BYTES];  // [buffer][K|V]
   __shared__ int s_sel;
 
@@ -223,6 +223,8 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_fp8_kernel(const AttnKern
         return i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
       };
 
+      // three waves share a SIMD (<= 168 VGPRs): all K operands are fetched up front, the V operands two
+      // at a time, the second pair under the first PV MFMAs
       i32x8 ka[4], va[4];
 #pragma unroll
       for (int n = 0; n < 4; ++n) ka[n] = read_k(n >> 1, n & 1);
@@ -231,9 +233,9 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_fp8_kernel(const AttnKern
       for (int t = 0; t < 2; ++t) {
         s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[2 * t], qf[0], zero16, 0, 0, 0, 0, 0, 0);
         s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[2 * t + 1], qf[1], s_acc[t], 0, 0, 0, 0, 0, 0);
-        va[2 * t] = read_v(2 * t);
-        va[2 * t + 1] = read_v(2 * t + 1);
       }
+      va[0] = read_v(0);
+      va[1] = read_v(1);
       if (k0 + BN > pe) {  // ragged last tile of a piece
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -275,8 +277,10 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_fwd_fp8_kernel(const AttnKern
           for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
       }
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
+      for (int mb = 0; mb < 4; ++mb) {
         o_acc[mb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va[mb], pb, o_acc[mb], 0, 0, 0, 0, 0, 0);
+        if (mb + 2 < 4) va[mb + 2] = read_v(mb + 2);
+      }
     }
     k0 = k1;
     pe = pe1;

@@ -19,9 +19,10 @@
 //
 // A single wavefront cannot keep the MFMA pipe busy (in-order issue, ~5 cycles between its VALU
 // instructions, LDS and MFMA latencies in series): throughput comes from several waves per SIMD
-// in different phases.  The kernel is therefore instantiated for 2 waves / SIMD (BN = 64, deep
-// operand prefetch, <= 256 VGPRs) and for 3 waves / SIMD (BN = 32, shallow prefetch, <= 168
-// VGPRs, 48 KB of LDS per workgroup).
+// in different phases.  The default instantiation runs 3 waves / SIMD: <= 168 VGPRs (shallow
+// operand prefetch) and 48 KB of LDS per workgroup (64-key tiles, K double buffered, ONE V slot that
+// is refilled under the score MFMAs and the softmax of the same tile).  Instantiations with 2 waves
+// / SIMD (deep prefetch, K and V double buffered) and with 32-key tiles are kept for comparison.
 //
 // Work decomposition: blockIdx -> (kv head, range slot, q tile, q head within the GQA group),
 // laid out so that the workgroups an XCD receives (blockIdx % 8) share a KV head and walk the
@@ -72,7 +73,7 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("" ::: "memory");
 }
 
-template <int NW, int BN, int NSTAGE, int OCC>
+template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
   constexpr int BM = 32 * NW;
   constexpr int TILE_BYTES = BN * ROW_BYTES;
@@ -83,7 +84,9 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   constexpr int DK = OCC >= 3 ? 4 : 8;     // K operands in flight
   constexpr int DV = OCC >= 3 ? 4 : 8;     // V operands in flight
   static_assert(LOADS >= 1 && NSTAGE >= 2 && NSTAGE <= 4, "bad tile configuration");
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[NSTAGE][2][TILE_BYTES];  // [stage][K|V]
+  static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");
+  // ring of NSTAGE (K tile, V tile) pairs, or in single-V mode K slot 0, K slot 1, V slot
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[VSINGLE ? 3 : 2 * NSTAGE][TILE_BYTES];
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -167,33 +170,33 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   const unsigned vvoff = (unsigned)row_in_tile0 * (unsigned)vs_t + (unsigned)(vchunk * 16);
   const bool small_strides = ks_t * (BN + 4) < (1l << 31) && vs_t * (BN + 4) < (1l << 31);
 
-  // Always TILE_LOADS load instructions per wave, so outstanding loads can be counted in tiles.
-  auto issue_tile = [&](int k0, int stage) {
-    unsigned char* kdst = &smem[stage][0][w * 1024];
-    unsigned char* vdst = &smem[stage][1][w * 1024];
+  // LOADS load instructions per wave per matrix per tile, always, so outstanding loads can be counted.
+  auto issue_mat = [&](int k0, unsigned char* tile_base, bool is_v) {
+    unsigned char* dst = tile_base + w * 1024;
+    const long st = is_v ? vs_t : ks_t;
+    const char* colp = is_v ? vcolp : kcolp;
+    const long d2 = is_v ? v2_delta : k2_delta;
     const bool interior = small_strides && (k0 + BN <= ke) && (k0 + BN <= k_split || k0 >= k_split);
     if (interior) {  // wave-uniform base + per-lane 32-bit offset
-      const bool second = k0 >= k_split;
-      const char* kb = kcolp + (long)k0 * ks_t + (second ? k2_delta : 0);
-      const char* vb = vcolp + (long)k0 * vs_t + (second ? v2_delta : 0);
+      const char* b = colp + (long)k0 * st + (k0 >= k_split ? d2 : 0);
+      const unsigned voff = is_v ? vvoff : kvoff;
 #pragma unroll
-      for (int j = 0; j < LOADS; ++j) {
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kb + (long)(4 * NW * j) * ks_t + kvoff),
-                                         LDS_PTR(void, kdst + j * NW * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vb + (long)(4 * NW * j) * vs_t + vvoff),
-                                         LDS_PTR(void, vdst + j * NW * 1024), 16, 0, 0);
-      }
+      for (int j = 0; j < LOADS; ++j)
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(b + (long)(4 * NW * j) * st + voff), LDS_PTR(void, dst + j * NW * 1024),
+                                         16, 0, 0);
     } else {  // ragged end of the range, or a tile that straddles the two key segments
+      const int chunk = is_v ? vchunk : kchunk;
 #pragma unroll
       for (int j = 0; j < LOADS; ++j) {
         const int row = min(k0 + row_in_tile0 + 4 * NW * j, ke - 1);
-        const bool second = row >= k_split;
-        const char* kp = kcolp + (long)row * ks_t + (second ? k2_delta : 0) + kchunk * 16;
-        const char* vp = vcolp + (long)row * vs_t + (second ? v2_delta : 0) + vchunk * 16;
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kp), LDS_PTR(void, kdst + j * NW * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vp), LDS_PTR(void, vdst + j * NW * 1024), 16, 0, 0);
+        const char* p = colp + (long)row * st + (row >= k_split ? d2 : 0) + chunk * 16;
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(p), LDS_PTR(void, dst + j * NW * 1024), 16, 0, 0);
       }
     }
+  };
+  auto issue_tile = [&](int k0, int stage) {
+    issue_mat(k0, &smem[2 * stage][0], false);
+    issue_mat(k0, &smem[2 * stage + 1][0], true);
   };
 
   // ---- per-lane LDS read bases ----
@@ -216,30 +219,44 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   const int n_tiles = (ke - ks + BN - 1) / BN;
+  if (VSINGLE) {
+    issue_mat(ks, &smem[0][0], false);
+  } else {
 #pragma unroll
-  for (int p = 0; p < NSTAGE - 1; ++p)
-    if (p < n_tiles) issue_tile(ks + p * BN, p);
+    for (int p = 0; p < NSTAGE - 1; ++p)
+      if (p < n_tiles) issue_tile(ks + p * BN, p);
+  }
   int stage = 0;
   for (int it = 0; it < n_tiles; ++it) {
     const int k0 = ks + it * BN;
-    // tile `it` must have landed; up to NSTAGE-2 younger tiles may still be in flight
-    const int younger = min(NSTAGE - 2, n_tiles - 1 - it);
-    if (NSTAGE >= 4 && younger == 2)
-      wait_vmcnt<2 * TILE_LOADS>();
-    else if (NSTAGE >= 3 && younger == 1)
-      wait_vmcnt<TILE_LOADS>();
-    else
+    if (VSINGLE) {
+      // single-V mode (48 KB of LDS, three workgroups per CU): K(it) was requested one iteration ago; V(it)
+      // is requested now, into the one V slot that PV(it-1) has just released, and lands under the score
+      // MFMAs and the softmax of this tile; a second barrier publishes it before PV(it).
       wait_vmcnt<0>();
-    __syncthreads();  // everybody's share landed; the stage read in the previous iteration is free again
-    if (it + NSTAGE - 1 < n_tiles) {
-      int st = stage + NSTAGE - 1;
-      if (st >= NSTAGE) st -= NSTAGE;
-      issue_tile(k0 + (NSTAGE - 1) * BN, st);
+      __syncthreads();
+      issue_mat(k0, &smem[2][0], true);
+      if (it + 1 < n_tiles) issue_mat(k0 + BN, &smem[(it + 1) & 1][0], false);
+    } else {
+      // tile `it` must have landed; up to NSTAGE-2 younger tiles may still be in flight
+      const int younger = min(NSTAGE - 2, n_tiles - 1 - it);
+      if (NSTAGE >= 4 && younger == 2)
+        wait_vmcnt<2 * TILE_LOADS>();
+      else if (NSTAGE >= 3 && younger == 1)
+        wait_vmcnt<TILE_LOADS>();
+      else
+        wait_vmcnt<0>();
+      __syncthreads();  // everybody's share landed; the stage read in the previous iteration is free again
+      if (it + NSTAGE - 1 < n_tiles) {
+        int st = stage + NSTAGE - 1;
+        if (st >= NSTAGE) st -= NSTAGE;
+        issue_tile(k0 + (NSTAGE - 1) * BN, st);
+      }
     }
-    const unsigned char* Kt = &smem[stage][0][0];
-    const unsigned char* Vt = &smem[stage][1][0];
+    const unsigned char* Kt = &smem[VSINGLE ? (it & 1) : 2 * stage][0];
+    const unsigned char* Vt = &smem[VSINGLE ? 2 : 2 * stage + 1][0];
     stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
-    if (!wave_on) continue;
+    if (!VSINGLE && !wave_on) continue;
 
     // LDS operand fetchers
     auto read_k = [&](int idx) -> bf16x8 {  // idx = 8t + kk
@@ -269,7 +286,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kbuf[idx % DK], qf[kk], kk == 0 ? zero16 : s_acc[t], 0, 0, 0);
       if (idx + DK < RK)
         kbuf[idx % DK] = read_k(idx + DK);
-      else if (idx + DK - RK < DV)
+      else if (!VSINGLE && idx + DK - RK < DV)
         vbuf[idx + DK - RK] = read_v(idx + DK - RK);
       if (DK == 8 && NT == 2 && idx == 7) __builtin_amdgcn_sched_barrier(0);
     }
@@ -318,6 +335,15 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
     // O^T[d][q] += V^T[d][key] P^T[key][q]; V operands run DV reads ahead
     __builtin_amdgcn_sched_barrier(0);
+    if (VSINGLE) {
+      if (it + 1 < n_tiles)
+        wait_vmcnt<LOADS>();  // V(it) landed; the K(it+1) loads issued after it may still be in flight
+      else
+        wait_vmcnt<0>();
+      __syncthreads();
+#pragma unroll
+      for (int p = 0; p < DV; ++p) vbuf[p] = read_v(p);
+    }
 #pragma unroll
     for (int p = 0; p < RV; ++p) {
       const int mb = p / NS, s = p % NS;
@@ -351,12 +377,14 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  if (a.block_m == 256)
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2>), dim3(grid), dim3(512), 0, stream, a);
-  else if (a.variant == 1)
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 32, 3, 3>), dim3(grid), dim3(256), 0, stream, a);
-  else
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2>), dim3(grid), dim3(256), 0, stream, a);
+  if (a.block_m == 256)  // 8 waves, 256 query rows, 2 waves / SIMD
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false>), dim3(grid), dim3(512), 0, stream, a);
+  else if (a.variant == 1)  // 32-key tiles, 3-stage ring, 3 waves / SIMD
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 32, 3, 3, false>), dim3(grid), dim3(256), 0, stream, a);
+  else if (a.variant == 2)  // 64-key tiles, double-buffered K and V, 2 waves / SIMD
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false>), dim3(grid), dim3(256), 0, stream, a);
+  else  // default: 64-key tiles, double-buffered K, single V slot, 3 waves / SIMD
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 

@@ -23,7 +23,7 @@ struct AttnKernArgs {
   int total_q, total_k, k_split;
   int n_ranges, ranges_mode, tiles_per_range;
   int block_m;  // q rows per workgroup: 128 (4 waves) or 256 (8 waves)
-  int variant;  // bf16 kernel instantiation: 0 = 2 waves/SIMD, 64-key tiles; 1 = 3 waves/SIMD, 32-key tiles
+  int variant;  // bf16 kernel instantiation, see launch_attn_fwd_bf16 (0 = default)
   int Hq, Hkv, G;
   int scale_chunk_tokens;
   unsigned total_wgs, per_xcd;

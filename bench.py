@@ -126,13 +126,18 @@ def fp8_leg(inp, core_fl, bf16_tflops, steps):
     the bf16 kernel's output on the same tensors."""
     import magi_attn as M
 
+    import math
+
     L, D = inp["L"], inp["D"]
     cache = inp["cache"]
-    q8, qs = M.quantize_fp8(inp["q"], L)
-    k8, ks = M.quantize_fp8(cache[..., :D], L)
-    v8, vs = M.quantize_fp8(cache[..., D:], L)
+    # power-of-two scales, softmax_scale * log2(e) folded into q before quantisation: the scales ride on the
+    # MFMA's block-scale operands and the kernel does no per-score multiply
+    q8, qs = M.quantize_fp8(inp["q"], L, premul=D ** -0.5 * math.log2(math.e), pow2_scales=True)
+    k8, ks = M.quantize_fp8(cache[..., :D], L, pow2_scales=True)
+    v8, vs = M.quantize_fp8(cache[..., D:], L, pow2_scales=True)
     out8 = torch.empty_like(inp["out"])
-    kw = dict(q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L, out=out8, return_lse=False)
+    kw = dict(q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L, out=out8, return_lse=False,
+              fp8_pow2_prescaled=True)
     M.range_attention(q8, k8, v8, inp["q_ranges"], inp["k_ranges"], L, **kw)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -30,6 +30,12 @@ extern "C" {
 #define MAGI_DTYPE_FP8_E4M3 1 /* OCP e4m3fn with per-(chunk, head) fp32 scales */
 
 /* how q_ranges / k_ranges are encoded */
+/* magi_attn_args.flags.  FP8_POW2_PRESCALED: every q/k/v scale is an exact power of two and q was multiplied by
+ * softmax_scale * log2(e) before quantisation (magi_quantize_fp8 with pow2_scales = 1 and that premul).  The
+ * scales then ride on the MFMA's block-scale operands and the kernel does no per-score multiply;
+ * softmax_scale is ignored. */
+#define MAGI_ATTN_FP8_POW2_PRESCALED 1
+
 #define MAGI_RANGES_PAIRS 0 /* int32 [n, 2]: range i = [r[2i], r[2i+1])          */
 #define MAGI_RANGES_CU 1    /* int32 [n + 1] cumulative: range i = [r[i], r[i+1]) */
 
@@ -98,7 +104,7 @@ typedef struct magi_attn_args {
   int32_t dtype;
   int32_t scale_chunk_tokens;
   float softmax_scale;
-  int32_t reserved;
+  int32_t flags; /* MAGI_ATTN_* bits */
 } magi_attn_args;
 
 int magi_attn_fwd(const magi_attn_args* args, void* stream);
@@ -165,13 +171,14 @@ int magi_apply_rotary(const void* x, const float* cos, const float* sin, void* y
 
 /*
  * Per-(chunk, head) absmax scales and OCP e4m3fn quantisation for the fp8 attention path:
- * scale[c, h] = max(absmax over tokens of chunk c and D, tiny) / 448;  y = sat_e4m3(x / scale).
+ * scale[c, h] = max(absmax over tokens of chunk c and D, tiny) * |premul| / 448, rounded UP to a power of two when
+ * pow2_scales is set;  y = sat_e4m3(x * premul / scale).
  * The quantiser follows the reference's only fp8 convention, div_clamp_to
  * (dit_module.py:364-384: clamp to +-448, saturating e4m3fn), without its bf16 intermediate.
  * x [T, H, D] bf16 with strides; y [T, H, D] fp8 contiguous; scales fp32 [ceil(T/chunk_tokens), H].
  */
 int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, float* scales, int32_t T,
-                      int32_t H, int32_t D, int32_t chunk_tokens, void* stream);
+                      int32_t H, int32_t D, int32_t chunk_tokens, float premul, int32_t pow2_scales, void* stream);
 
 #ifdef __cplusplus
 }

@@ -111,6 +111,7 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.Hkv = p->Hkv;
   a.G = p->Hq / p->Hkv;
   a.scale_chunk_tokens = p->scale_chunk_tokens;
+  a.flags = p->flags;
   const double total = (double)p->Hq * p->n_ranges * a.tiles_per_range;
   if (total > 2.0e9) return fail(MAGI_EINVAL, "magi_attn_fwd: grid too large (%.3g workgroups)", total);
   a.total_wgs = (unsigned)total;
@@ -210,16 +211,17 @@ int magi_apply_rotary(const void* x, const float* cos, const float* sin, void* y
 }
 
 int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, float* scales, int32_t T,
-                      int32_t H, int32_t D, int32_t chunk_tokens, void* stream) {
+                      int32_t H, int32_t D, int32_t chunk_tokens, float premul, int32_t pow2_scales, void* stream) {
   if (D != 128) return fail(MAGI_ENOSYS, "magi_quantize_fp8: head_dim %d not implemented (128 only)", D);
   if (T < 0 || H < 0 || chunk_tokens <= 0) return fail(MAGI_EINVAL, "magi_quantize_fp8: bad size");
+  if (!(premul == premul) || premul == 0.f) return fail(MAGI_EINVAL, "magi_quantize_fp8: premul must be finite and non-zero");
   if (T == 0 || H == 0) return MAGI_OK;
   if (!x || !y || !scales) return fail(MAGI_EINVAL, "magi_quantize_fp8: NULL pointer");
   if (x_stride_t % 8 || x_stride_h % 8 || !aligned16(x) || !aligned16(y))
     return fail(MAGI_EINVAL, "magi_quantize_fp8: rows must be 16-byte aligned");
   hipError_t e = magi::launch_quantize_fp8(static_cast<const char*>(x), x_stride_t * 2, x_stride_h * 2,
-                                           static_cast<char*>(y), scales, T, H, chunk_tokens,
-                                           static_cast<hipStream_t>(stream));
+                                           static_cast<char*>(y), scales, T, H, chunk_tokens, premul,
+                                           pow2_scales, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_quantize_fp8 launch");
   return MAGI_OK;
 }

@@ -54,6 +54,7 @@ __device__ __forceinline__ void load_range(const int* r, int mode, int i, int to
   e = max(s, min(e, total));
 }
 
+template <bool POW2>
 __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKernArgs a) {
   __shared__ __attribute__((aligned(1024))) unsigned char smem[2][2][TILE_BYTES];  // [buffer][K|V]
   __shared__ int s_sel;
@@ -180,8 +181,18 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o_acc[mb][v] = 0.f;
-  float m_run = -__builtin_inff();  // running max in scaled log2 units
+  // Running maximum in exp2-exponent units.  In the general mode it starts at -inf; in the power-of-two mode
+  // the score MFMAs accumulate onto neg_m = shift - m in all 16 registers (a lane's registers all belong to one
+  // query), so they deliver the exp2 exponent directly and a tile only pays for a correction when it raises a
+  // row's maximum; there m starts at 0 and the first tile sets it.
+  float m_run = POW2 ? 0.f : -__builtin_inff();
   float l_run = 0.f;
+  f32x16 neg_m;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) neg_m[v] = 0.f;
+  float cur_shift = 0.f;
+  bool first = true;
+  const int e_q = (__builtin_bit_cast(int, q_sc) >> 23) & 0xff;  // E8M0 code of the (power-of-two) query scale
   const bool wave_on = (q0 + 32 * w) < qe;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const float c_q = a.scale_log2 * q_sc;  // softmax scale * log2(e) * q scale
@@ -223,19 +234,42 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         return i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
       };
 
-      // three waves share a SIMD (<= 168 VGPRs): all K operands are fetched up front, the V operands two
-      // at a time, the second pair under the first PV MFMAs
-      i32x8 ka[4], va[4];
-#pragma unroll
-      for (int n = 0; n < 4; ++n) ka[n] = read_k(n >> 1, n & 1);
+      // three waves share a SIMD (<= 168 VGPRs): K operands are fetched two at a time, V operands two at a time,
+      // the second pair under the first PV MFMAs
+      i32x8 ka[2], va[2];
       f32x16 s_acc[2];
+      i32x8 pb;
+      float psum = 0.f;
+      ka[0] = read_k(0, 0);
+      ka[1] = read_k(0, 1);
+      if constexpr (POW2) {
+        const int e_k = (__builtin_bit_cast(int, k_sc) >> 23) & 0xff;
+        if (shift != cur_shift) {  // a new scale chunk (wave-uniform): re-base the accumulator offset
+          const float ds = shift - cur_shift;
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[2 * t], qf[0], zero16, 0, 0, 0, 0, 0, 0);
-        s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[2 * t + 1], qf[1], s_acc[t], 0, 0, 0, 0, 0, 0);
+          for (int v = 0; v < 16; ++v) neg_m[v] += ds;
+          cur_shift = shift;
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[0], qf[0], neg_m, 0, 0, 0, e_k, 0, e_q);
+          if (t == 0) ka[0] = read_k(1, 0);
+          s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[1], qf[1], s_acc[t], 0, 0, 0, e_k, 0, e_q);
+          if (t == 0) ka[1] = read_k(1, 1);
+        }
+      } else {
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[0], qf[0], zero16, 0, 0, 0, 0, 0, 0);
+          if (t == 0) ka[0] = read_k(1, 0);
+          s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[1], qf[1], s_acc[t], 0, 0, 0, 0, 0, 0);
+          if (t == 0) ka[1] = read_k(1, 1);
+        }
       }
-      va[0] = read_v(0);
-      va[1] = read_v(1);
+      if (!POW2) {  // the power-of-two mode keeps 16 registers for neg_m and fetches V after the softmax instead
+        va[0] = read_v(0);
+        va[1] = read_v(1);
+      }
       if (k0 + BN > pe) {  // ragged last tile of a piece
 #pragma unroll
         for (int t = 0; t < 2; ++t)
@@ -251,35 +285,75 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
 #pragma unroll
         for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[t][v]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
-      const float m_new = fmaxf(m_run, mx * c);
-      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-      const float mc = m_new - shift;
-      m_run = m_new;
-      float psum = 0.f;
-      i32x8 pb;
+      if constexpr (POW2) {
+        // s_acc already holds exponent - m_run + shift; a value above `shift` is a new row maximum
+        const float over = mx - shift;
+        const bool raise = first || over > 0.f;
+        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+          const float delta = raise ? over : 0.f;
+          const float alpha = __builtin_amdgcn_exp2f(-delta);
+          m_run += delta;
+          l_run *= alpha;
 #pragma unroll
-      for (int n = 0; n < 8; ++n) {  // dword n = slots 4n .. 4n+3 = s_acc[n >> 2][4 (n & 3) .. +3]
-        const float p0 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 0] * c - mc);
-        const float p1 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 1] * c - mc);
-        const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2] * c - mc);
-        const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3] * c - mc);
-        psum += (p0 + p1) + (p2 + p3);
-        int u = 0;
-        u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
-        u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
-        pb[n] = u;
+          for (int v = 0; v < 16; ++v) neg_m[v] -= delta;
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) s_acc[t][v] -= delta;
+          if (!first) {
+#pragma unroll
+            for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+              for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+          }
+        }
+        first = false;
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {  // dword n = slots 4n .. 4n+3 = s_acc[n >> 2][4 (n & 3) .. +3]
+          const float p0 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 0]);
+          const float p1 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 1]);
+          const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2]);
+          const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3]);
+          psum += (p0 + p1) + (p2 + p3);
+          int u = 0;
+          u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
+          u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
+          pb[n] = u;
+        }
+        l_run += psum * unshift;
+      } else {
+        const float m_new = fmaxf(m_run, mx * c);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        const float mc = m_new - shift;
+        m_run = m_new;
+#pragma unroll
+        for (int n = 0; n < 8; ++n) {
+          const float p0 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 0] * c - mc);
+          const float p1 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 1] * c - mc);
+          const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2] * c - mc);
+          const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3] * c - mc);
+          psum += (p0 + p1) + (p2 + p3);
+          int u = 0;
+          u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
+          u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
+          pb[n] = u;
+        }
+        l_run = l_run * alpha + psum * unshift;
+        if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+        }
       }
-      l_run = l_run * alpha + psum * unshift;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+      if (POW2) {
+        va[0] = read_v(0);
+        va[1] = read_v(1);
       }
 #pragma unroll
-      for (int mb = 0; mb < 4; ++mb) {
-        o_acc[mb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va[mb], pb, o_acc[mb], 0, 0, 0, 0, 0, 0);
-        if (mb + 2 < 4) va[mb + 2] = read_v(mb + 2);
+      for (int mb = 0; mb < 4; ++mb) {  // two V operands in flight, in alternating registers
+        o_acc[mb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va[mb & 1], pb, o_acc[mb], 0, 0, 0, 0, 0, 0);
+        if (mb + 2 < 4) va[mb & 1] = read_v(mb + 2);
       }
     }
     k0 = k1;
@@ -344,14 +418,21 @@ __global__ __launch_bounds__(QT) void absmax_kernel(const char* x, long xs_t, lo
   }
 }
 
-__global__ __launch_bounds__(QT) void finalize_scales_kernel(float* scales, int n) {
+__global__ __launch_bounds__(QT) void finalize_scales_kernel(float* scales, int n, float premul, int pow2) {
   const int i = blockIdx.x * QT + threadIdx.x;
-  if (i < n) scales[i] = fmaxf(scales[i] / 448.f, 1e-12f);
+  if (i >= n) return;
+  float f = fmaxf(scales[i] * fabsf(premul) / 448.f, 1e-12f);
+  if (pow2) {  // round up to a power of two
+    unsigned b = __builtin_bit_cast(unsigned, f);
+    b = ((b >> 23) + ((b & 0x7fffffu) ? 1u : 0u)) << 23;
+    f = __builtin_bit_cast(float, b);
+  }
+  scales[i] = f;
 }
 
 // one thread per 8 elements
 __global__ __launch_bounds__(QT) void quantize_kernel(const char* x, long xs_t, long xs_h, char* y, const float* scales,
-                                                      int T, int H, int chunk_tokens) {
+                                                      int T, int H, int chunk_tokens, float premul) {
   const long gid = (long)blockIdx.x * QT + threadIdx.x;
   const long row = gid >> 4;
   const int part = (int)(gid & 15);
@@ -366,7 +447,7 @@ __global__ __launch_bounds__(QT) void quantize_kernel(const char* x, long xs_t, 
     fv[2 * j + 1] = __builtin_bit_cast(float, v[j] & 0xffff0000u);
   }
 #pragma unroll
-  for (int j = 0; j < 8; ++j) fv[j] = fminf(fmaxf(fv[j] / sc, -448.f), 448.f);
+  for (int j = 0; j < 8; ++j) fv[j] = fminf(fmaxf(fv[j] * premul / sc, -448.f), 448.f);
   u32x2 o;
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -382,12 +463,15 @@ __global__ __launch_bounds__(QT) void quantize_kernel(const char* x, long xs_t, 
 
 hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  hipLaunchKernelGGL(attn_fwd_fp8_kernel, dim3(grid), dim3(64 * NW), 0, stream, a);
+  if (a.flags & 1)
+    hipLaunchKernelGGL(attn_fwd_fp8_kernel<true>, dim3(grid), dim3(64 * NW), 0, stream, a);
+  else
+    hipLaunchKernelGGL(attn_fwd_fp8_kernel<false>, dim3(grid), dim3(64 * NW), 0, stream, a);
   return hipGetLastError();
 }
 
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
-                               int chunk_tokens, hipStream_t stream) {
+                               int chunk_tokens, float premul, int pow2_scales, hipStream_t stream) {
   const int n_chunks = (T + chunk_tokens - 1) / chunk_tokens;
   const int n = n_chunks * H;
   hipLaunchKernelGGL(fill_zero_kernel, dim3((n + QT - 1) / QT), dim3(QT), 0, stream, (unsigned*)scales, n);
@@ -396,10 +480,10 @@ hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, 
   slices = max(1, min(slices, 256));
   hipLaunchKernelGGL(absmax_kernel, dim3(slices, H, n_chunks), dim3(QT), 0, stream, x, x_stride_t, x_stride_h,
                      (unsigned*)scales, T, H, chunk_tokens);
-  hipLaunchKernelGGL(finalize_scales_kernel, dim3((n + QT - 1) / QT), dim3(QT), 0, stream, scales, n);
+  hipLaunchKernelGGL(finalize_scales_kernel, dim3((n + QT - 1) / QT), dim3(QT), 0, stream, scales, n, premul, pow2_scales);
   const long threads = (long)T * H * 16;
   hipLaunchKernelGGL(quantize_kernel, dim3((unsigned)((threads + QT - 1) / QT)), dim3(QT), 0, stream, x, x_stride_t,
-                     x_stride_h, y, scales, T, H, chunk_tokens);
+                     x_stride_h, y, scales, T, H, chunk_tokens, premul);
   return hipGetLastError();
 }
 

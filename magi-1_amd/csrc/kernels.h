@@ -26,6 +26,7 @@ struct AttnKernArgs {
   int variant;  // bf16 kernel instantiation, see launch_attn_fwd_bf16 (0 = default)
   int Hq, Hkv, G;
   int scale_chunk_tokens;
+  int flags;
   unsigned total_wgs, per_xcd;
   float scale_log2;  // softmax_scale * log2(e)
 };
@@ -61,6 +62,6 @@ hipError_t launch_head_norm(const char* x, long x_stride_t, long x_stride_h, con
 hipError_t launch_rotary(const void* x, const float* cos, const float* sin, void* y, int B, int S, int H, int D,
                          int R2, int is_bf16, hipStream_t stream);
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
-                               int chunk_tokens, hipStream_t stream);
+                               int chunk_tokens, float premul, int pow2_scales, hipStream_t stream);
 
 }  // namespace magi

@@ -18,6 +18,7 @@ MAGI_RANGES_CU = 1
 MAGI_NORM_LAYERNORM_1P = 0
 MAGI_NORM_RMSNORM_1P = 1
 MAGI_NORM_NONE = 2
+MAGI_ATTN_FP8_POW2_PRESCALED = 1
 
 
 class MagiError(RuntimeError):
@@ -40,7 +41,7 @@ class AttnArgs(C.Structure):
         ("max_seqlen_q", C.c_int32), ("max_seqlen_k", C.c_int32),
         ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32),
         ("dtype", C.c_int32), ("scale_chunk_tokens", C.c_int32),
-        ("softmax_scale", C.c_float), ("reserved", C.c_int32),
+        ("softmax_scale", C.c_float), ("flags", C.c_int32),
     ]
 
 
@@ -85,7 +86,7 @@ def lib() -> C.CDLL:
                                         C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
         l.magi_apply_rotary.restype = C.c_int
         l.magi_quantize_fp8.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32,
-                                        C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
+                                        C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_int32, C.c_void_p]
         l.magi_quantize_fp8.restype = C.c_int
         _lib = l
     return _lib

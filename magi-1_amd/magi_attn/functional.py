@@ -65,6 +65,7 @@ def range_attention(
     k_scale: Optional[torch.Tensor] = None,
     v_scale: Optional[torch.Tensor] = None,
     scale_chunk_tokens: int = 0,
+    fp8_pow2_prescaled: bool = False,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = True,
     zero_init: bool = True,
@@ -125,6 +126,7 @@ def range_attention(
     a.dtype = _dtype_code(q)
     a.scale_chunk_tokens = int(scale_chunk_tokens)
     a.softmax_scale = 0.0 if softmax_scale is None else float(softmax_scale)
+    a.flags = L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0
     with torch.cuda.device(q.device):
         L.check(L.lib().magi_attn_fwd(C.byref(a), _stream()))
     return out, lse
@@ -254,9 +256,13 @@ def head_norm(x: torch.Tensor, gamma, beta, eps: float = 1e-6, norm_kind: int = 
     return y
 
 
-def quantize_fp8(x: torch.Tensor, chunk_tokens: int):
+def quantize_fp8(x: torch.Tensor, chunk_tokens: int, premul: float = 1.0, pow2_scales: bool = False):
     """x [T, H, 128] bf16 (strided heads allowed) -> (y [T, H, 128] float8_e4m3fn, scales [ceil(T/chunk), H] fp32)
-    with x ~= y * scales[t // chunk_tokens, h]: per-(chunk, head) absmax / 448, saturating OCP e4m3fn."""
+    with x * premul ~= y * scales[t // chunk_tokens, h]: per-(chunk, head) absmax * |premul| / 448 (rounded up to a
+    power of two with pow2_scales), saturating OCP e4m3fn.
+
+    For the fast attention mode quantise q with premul = softmax_scale * log2(e) and q, k, v with pow2_scales,
+    then pass fp8_pow2_prescaled=True to range_attention."""
     _check_thd(x, "x")
     if x.dtype != torch.bfloat16:
         raise TypeError("x must be bf16")
@@ -266,5 +272,5 @@ def quantize_fp8(x: torch.Tensor, chunk_tokens: int):
     scales = torch.empty((n_chunks, H), dtype=torch.float32, device=x.device)
     with torch.cuda.device(x.device):
         L.check(L.lib().magi_quantize_fp8(x.data_ptr(), x.stride(0), x.stride(1), y.data_ptr(), scales.data_ptr(), T, H, D,
-                                          int(chunk_tokens), _stream()))
+                                          int(chunk_tokens), float(premul), int(pow2_scales), _stream()))
     return y, scales

@@ -381,24 +381,28 @@ def quantize_e4m3(x: torch.Tensor, scale: torch.Tensor, via_bf16: bool = False) 
     return y.to(torch.float8_e4m3fn)
 
 
-def per_head_chunk_scales(x: torch.Tensor, chunk_token_nums: int) -> torch.Tensor:
-    """absmax over (chunk tokens, D) per head / 448 -> [n_chunks, H] fp32 (>= tiny)."""
+def per_head_chunk_scales(x: torch.Tensor, chunk_token_nums: int, premul: float = 1.0, pow2: bool = False) -> torch.Tensor:
+    """absmax over (chunk tokens, D) per head * |premul| / 448 -> [n_chunks, H] fp32 (>= tiny); with pow2 the
+    scale is rounded up to the next power of two."""
     T, H, D = x.shape
     n = (T + chunk_token_nums - 1) // chunk_token_nums
     out = torch.empty(n, H, dtype=torch.float32)
     for c in range(n):
         blk = x[c * chunk_token_nums:(c + 1) * chunk_token_nums].float()
-        out[c] = blk.abs().amax(dim=(0, 2)) / FP8_MAX
-    return out.clamp_min(1e-12)
+        out[c] = blk.abs().amax(dim=(0, 2)) * torch.tensor(abs(premul), dtype=torch.float32) / FP8_MAX
+    out = out.clamp_min(1e-12)
+    if pow2:
+        out = torch.exp2(torch.ceil(torch.log2(out.double()))).float()
+    return out
 
 
-def quantize_per_head_chunk(x: torch.Tensor, chunk_token_nums: int):
-    """-> (x_fp8 [T,H,D] float8_e4m3fn, scales [n_chunks,H] fp32) with x ~= x_fp8 * scale."""
-    scales = per_head_chunk_scales(x, chunk_token_nums)
+def quantize_per_head_chunk(x: torch.Tensor, chunk_token_nums: int, premul: float = 1.0, pow2: bool = False):
+    """-> (x_fp8 [T,H,D] float8_e4m3fn, scales [n_chunks,H] fp32) with x * premul ~= x_fp8 * scale."""
+    scales = per_head_chunk_scales(x, chunk_token_nums, premul, pow2)
     T = x.shape[0]
     idx = torch.arange(T) // chunk_token_nums
     s = scales[idx][:, :, None]
-    return quantize_e4m3(x, s), scales
+    return quantize_e4m3(x.float() * torch.tensor(premul, dtype=torch.float32), s), scales
 
 
 def dequantize_per_head_chunk(x8: torch.Tensor, scales: torch.Tensor, chunk_token_nums: int) -> torch.Tensor:

@@ -70,6 +70,37 @@ def test_fp8_attention_parity(dev, L, dn, sp, Hq, Hkv, C):
     assert (lse.cpu() - lse_ref).abs().max() < 1e-3
 
 
+@pytest.mark.parametrize("L,dn,sp,Hq,Hkv,C", [(128, 1, 0, 1, 1, 128), (200, 3, 1, 6, 2, 200), (77, 2, 2, 3, 1, 50),
+                                              (1536, 3, 0, 24, 8, 1536)])
+def test_fp8_pow2_prescaled_mode(dev, L, dn, sp, Hq, Hkv, C):
+    """Fast mode: power-of-two scales on the MFMA block-scale operands, softmax_scale * log2(e) folded into q at
+    quantisation.  Quantiser bit-exact with the oracle's; attention within the same stated tolerance."""
+    import math
+
+    cs = 128 ** -0.5 * math.log2(math.e)
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=6234 + L)
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    q8, qs = M.quantize_fp8(q.to(dev), C, premul=cs, pow2_scales=True)
+    k8, ks = M.quantize_fp8(k.to(dev), C, pow2_scales=True)
+    v8, vs = M.quantize_fp8(v.to(dev), C, pow2_scales=True)
+    q8r, qsr = O.quantize_per_head_chunk(q, C, cs, True)
+    assert torch.equal(qs.cpu(), qsr) and torch.equal(q8.cpu().view(torch.uint8), q8r.view(torch.uint8))
+    assert torch.all(torch.frexp(ks.cpu())[0] == 0.5) and torch.all(torch.frexp(qs.cpu())[0] == 0.5)  # powers of two
+    tq, tk = torch.tensor(qr, device=dev), torch.tensor(kr, device=dev)
+    out, lse = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=C,
+                                 fp8_pow2_prescaled=True)
+    err, cos = _per_head(out, O.range_attention(q, k, v, qr, kr))
+    assert err <= 2 ** -5 * v.float().abs().max().item() and cos >= 0.998, (err, cos)
+    # dequantised inputs (q side carries the folded scale, so the oracle runs with scale 1 in base 2)
+    qd = O.dequantize_per_head_chunk(q8.cpu(), qs.cpu(), C) / cs * 128 ** -0.5
+    kd = O.dequantize_per_head_chunk(k8.cpu(), ks.cpu(), C)
+    vd = O.dequantize_per_head_chunk(v8.cpu(), vs.cpu(), C)
+    err, cos = _per_head(out, O.range_attention(qd, kd, vd, qr, kr, softmax_scale=1.0))
+    assert err <= 4e-2 and cos >= 0.9995, (err, cos)
+    lse_ref = O.range_attention_lse(qd, kd, vd, qr, kr, softmax_scale=1.0)
+    assert (lse.cpu() - lse_ref).abs().max() < 1e-3
+
+
 def test_fp8_uneven_scales_and_two_segments(dev):
     """Chunks with very different magnitudes (the per-chunk scales must be honoured, including the
     relative V scale folded into the exponent) and a key axis split over two buffers."""
@@ -91,6 +122,18 @@ def test_fp8_uneven_scales_and_two_segments(dev):
     split = sp * L + 40
     out2, _ = M.range_attention(q8, k8[:split], v8[:split], tq, tk, L, k2=k8[split:].clone(), v2=v8[split:].clone(),
                                 k_split=split, **kw)
+    # the same uneven chunks through the power-of-two mode
+    import math
+    cs = 128 ** -0.5 * math.log2(math.e)
+    q8p, qsp = M.quantize_fp8(q.to(dev), L, premul=cs, pow2_scales=True)
+    k8p, ksp = M.quantize_fp8(k.to(dev), L, pow2_scales=True)
+    v8p, vsp = M.quantize_fp8(v.to(dev), L, pow2_scales=True)
+    out3, _ = M.range_attention(q8p, k8p, v8p, tq, tk, L, q_scale=qsp, k_scale=ksp, v_scale=vsp, scale_chunk_tokens=L,
+                                fp8_pow2_prescaled=True)
+    qd = O.dequantize_per_head_chunk(q8p.cpu(), qsp.cpu(), L) / cs * 128 ** -0.5
+    deq3 = O.range_attention(qd, O.dequantize_per_head_chunk(k8p.cpu(), ksp.cpu(), L),
+                             O.dequantize_per_head_chunk(v8p.cpu(), vsp.cpu(), L), qr, kr, softmax_scale=1.0)
+    assert ((out3.double().cpu() - deq3.double()).abs().max() / deq3.abs().max()).item() <= 4e-2
     # the split moves tile boundaries (a piece ends at the split), so rounding may differ by a bf16 ulp or two
     assert (out2.float() - out.float()).abs().max().item() <= 4e-2 * deq.abs().max().item()
 

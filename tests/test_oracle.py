@@ -1,7 +1,9 @@
 """Pins of the CPU oracle: each restated function is checked against something other than
 its own formula (closed forms, library routines, brute force, invariants, and the vectors the
 reference keeps in comments)."""
+import json
 import math
+import os
 
 import numpy as np
 import pytest
@@ -9,6 +11,8 @@ import torch
 import torch.nn.functional as F
 
 from oracle import magi_oracle as O
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
 
 
 # ----------------------------------------------------------------------------- rope table
@@ -284,18 +288,36 @@ def test_kv_cache_model_against_list_of_chunks():
 
 # ----------------------------------------------------------------------------- chunk-window arithmetic
 def test_generate_sequences_reference_comment_examples():
-    # the four worked examples kept next to the function in the reference (video_generate.py:139-161)
-    assert O.generate_sequences(8, 8, 0) == (
-        [0, 0, 0, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5, 6, 7], [1, 2, 3, 4, 5, 6, 7, 8, 8, 8, 8, 8, 8, 8, 8],
-        [0, 0, 0, 0, 0, 0, 0, 0, 1, 2, 3, 4, 5, 6, 7], [1, 2, 3, 4, 5, 6, 7, 8, 8, 8, 8, 8, 8, 8, 8])
-    assert O.generate_sequences(8, 4, 0) == (
-        [0, 0, 0, 0, 1, 2, 3, 4, 5, 6, 7], [1, 2, 3, 4, 5, 6, 7, 8, 8, 8, 8],
-        [0, 0, 0, 0, 0, 0, 0, 0, 1, 2, 3], [1, 2, 3, 4, 4, 4, 4, 4, 4, 4, 4])
-    assert O.generate_sequences(8, 4, 2) == (
-        [2, 2, 2, 2, 3, 4, 5, 6, 7], [3, 4, 5, 6, 7, 8, 8, 8, 8],
-        [0, 0, 0, 0, 0, 0, 1, 2, 3], [1, 2, 3, 4, 4, 4, 4, 4, 4])
-    assert O.generate_sequences(8, 1, 0) == (
-        [0, 1, 2, 3, 4, 5, 6, 7], [1, 2, 3, 4, 5, 6, 7, 8], [0] * 8, [1] * 8)
+    # the four worked examples kept next to the function in the reference (video_generate.py:139-161),
+    # held as data in tests/golden/generate_sequences_examples.json
+    with open(os.path.join(GOLDEN, "generate_sequences_examples.json")) as f:
+        examples = json.load(f)
+    assert len(examples) == 4
+    for e in examples:
+        got = O.generate_sequences(e["chunk_num"], e["window_size"], e["chunk_offset"])
+        assert got == (e["clip_start"], e["clip_end"], e["t_start"], e["t_end"]), e
+
+
+def test_layer_small_fixture_matches_oracle():
+    # the frozen small layer pass: the oracle must still produce it from the stored inputs
+    z = np.load(os.path.join(GOLDEN, "layer_small.npz"))
+    bf = lambda a: torch.from_numpy(a.view(np.int16).copy()).view(torch.bfloat16)
+    T, H, W, prefix, dn, Hq, Hkv, D = (int(x) for x in z["dims"])
+    L = T * H * W
+    assert np.array_equal(z["rope"], O.rope_for_forward(dn * T, H, W, prefix, dn).numpy())
+    assert np.array_equal(z["q_ranges"], O.q_ranges_for(dn, L)) and np.array_equal(z["k_ranges"], O.default_kvrange(prefix, dn, L))
+    q, kv = O.prologue(bf(z["q_raw"]), bf(z["k_raw"]), bf(z["v_raw"]), torch.from_numpy(z["rope"]),
+                       *(torch.from_numpy(z[n]) for n in ("gq", "bq", "gk", "bk")))
+    assert torch.equal(q, bf(z["q"])) and torch.equal(kv, bf(z["kv"]))
+    cache = torch.cat([bf(z["prefix_kv"]), kv], 0)
+    out = O.range_attention(q, cache[..., :D], cache[..., D:], z["q_ranges"], z["k_ranges"])
+    assert torch.allclose(out.float(), torch.from_numpy(z["out"]), atol=1e-5, rtol=0)
+    # independent check of the frozen output: fp64 brute force over the same stored tensors
+    ref = O.brute_attention_fp64(q, cache[..., :D], cache[..., D:], z["q_ranges"], z["k_ranges"])
+    assert torch.allclose(torch.from_numpy(z["out"]).double(), ref, atol=2e-5, rtol=0)
+    xout = O.varlen_cross_attention(q, bf(z["xk"]), bf(z["xv"]), z["cu_q"], z["cu_k"])
+    assert torch.allclose(xout.float(), torch.from_numpy(z["xout"]), atol=1e-5, rtol=0)
+    assert torch.count_nonzero(torch.from_numpy(z["xout"])[L:]) == 0  # empty text segment -> zeros
 
 
 def test_kvrange_tables_hand_derived():

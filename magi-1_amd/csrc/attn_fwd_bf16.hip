@@ -30,6 +30,8 @@
 // first.  Fully masked key tiles never exist: a rectangle is walked from k_start to k_end only.
 #include "kernels.h"
 
+#include <type_traits>
+
 namespace magi {
 namespace {
 
@@ -39,6 +41,7 @@ typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 
@@ -66,6 +69,15 @@ __device__ __forceinline__ void load_range(const int* r, int mode, int i, int to
   e = max(s, min(e, total));
 }
 
+// f(integral_constant<int, I>) for I = B .. E-1, unrolled at compile time
+template <int B, int E, class F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (B < E) {
+    f(std::integral_constant<int, B>{});
+    static_for<B + 1, E>(f);
+  }
+}
+
 // s_waitcnt vmcnt(N), leaving the other counters alone
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
@@ -73,7 +85,26 @@ __device__ __forceinline__ void wait_vmcnt() {
   asm volatile("" ::: "memory");
 }
 
-template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE>
+// wave-wide max of the two half-waves' values (lane i and lane i + 32 hold the same query)
+__device__ __forceinline__ float half_swap_max(float x) {
+  const unsigned u = __builtin_bit_cast(unsigned, x);
+  const u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
+}
+
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
+// p0 + p1 + acc for a packed pair of bf16 values
+__device__ __forceinline__ float pair_sum(unsigned pk, float acc) {
+  const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), one, acc, false);
+}
+
+template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool PIPE = false>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
   constexpr int BM = 32 * NW;
   constexpr int TILE_BYTES = BN * ROW_BYTES;
@@ -85,8 +116,10 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   constexpr int DV = OCC >= 3 ? 4 : 8;     // V operands in flight
   static_assert(LOADS >= 1 && NSTAGE >= 2 && NSTAGE <= 4, "bad tile configuration");
   static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");
+  static_assert(!PIPE || (NSTAGE == 2 && BN == 64 && !VSINGLE), "pipelined loop: 64-key tiles, two K slots and two V slots");
   // ring of NSTAGE (K tile, V tile) pairs, or in single-V mode K slot 0, K slot 1, V slot
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[VSINGLE ? 3 : 2 * NSTAGE][TILE_BYTES];
+  // (pipelined loop: K slots 0, 1 and V slots 2, 3)
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[PIPE ? 1 : VSINGLE ? 3 : 2 * NSTAGE][PIPE ? 16 : TILE_BYTES];
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -177,13 +210,18 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
     const char* colp = is_v ? vcolp : kcolp;
     const long d2 = is_v ? v2_delta : k2_delta;
     const bool interior = small_strides && (k0 + BN <= ke) && (k0 + BN <= k_split || k0 >= k_split);
-    if (interior) {  // wave-uniform base + per-lane 32-bit offset
+    if (interior) {
+      // Buffer-addressed direct loads: scalar base (the tile's first row) in the resource descriptor, one
+      // loop-invariant 32-bit lane offset, the row group of load j in the scalar offset.  This form costs the
+      // SIMD next to nothing to issue; the 64-bit-address-per-lane form of the same load stalls it for well
+      // over a hundred cycles per instruction.
       const char* b = colp + (long)k0 * st + (k0 >= k_split ? d2 : 0);
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)b, 0, 0x7fffffff, 0x00020000);
       const unsigned voff = is_v ? vvoff : kvoff;
 #pragma unroll
       for (int j = 0; j < LOADS; ++j)
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(b + (long)(4 * NW * j) * st + voff), LDS_PTR(void, dst + j * NW * 1024),
-                                         16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * NW * 1024), 16, voff,
+                                                 (int)((unsigned)(4 * NW * j) * (unsigned)st), 0, 0);
     } else {  // ragged end of the range, or a tile that straddles the two key segments
       const int chunk = is_v ? vchunk : kchunk;
 #pragma unroll
@@ -219,6 +257,184 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   const int n_tiles = (ke - ks + BN - 1) / BN;
+  if constexpr (PIPE) {
+    // Software-pipelined loop.  Iteration `it` runs, in ONE basic block, the score MFMAs of tile it+1, the
+    // exp2 / pack / row-sum work of tile it, the PV MFMAs of tile it and the row max of tile it+1, cut into
+    // 32 chunks of one MFMA + its operand reads + a few VALU instructions each (scheduling barriers pin the
+    // chunks), so that the VALU work issues in the shadow of the MFMAs of the same wave.  The lazy rescale of
+    // O and the tail mask sit between iterations.  K(t) lives in K slot t & 1, V(t) in V slot t & 1; the loads
+    // for K(it+2) and V(it+1) are issued at the top of iteration it and have the whole iteration to land.
+    // The four slots are four separate LDS objects and the loop is unrolled by two so that every access names
+    // its slot statically: the compiler then knows that the operand reads of an iteration never touch the
+    // slots the in-flight direct loads write, and does not make the reads wait for those loads.
+    __shared__ __attribute__((aligned(1024))) unsigned char sK0[TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char sK1[TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char sV0[TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char sV1[TILE_BYTES];
+    auto read_k = [&](const unsigned char* Kt, int idx) -> bf16x8 {  // idx = 8t + kk
+      return *LDS_PTR(const bf16x8, Kt + ((base_k ^ ((idx & 7) << 5)) + (idx >> 3) * 32 * ROW_BYTES));
+    };
+    auto read_v = [&](const unsigned char* Vt, int p) -> bf16x8 {  // p = 4 * slab + mb
+      const int mb = p & 3, sl = p >> 2;
+      const int bv = base_v ^ (mb << 6);
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * sl) * ROW_BYTES)));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * sl + 8) * ROW_BYTES)));
+      const s16x8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+      return __builtin_bit_cast(bf16x8, va);
+    };
+    constexpr int PD = 4;  // operand reads in flight (2 .. 8 measure the same)
+    f32x16 sA[2], sB[2];   // scores of even / odd tiles
+    float m_new, alpha;
+
+    // ---- prologue: K(0) -> scores of tile 0 and their row max ----
+    issue_mat(ks, sK0, false);
+    wait_vmcnt<0>();
+    __syncthreads();
+    if (n_tiles > 1) issue_mat(ks + BN, sK1, false);
+    issue_mat(ks, sV0, true);
+    {
+      bf16x8 kbuf[PD];
+#pragma unroll
+      for (int idx = 0; idx < PD; ++idx) kbuf[idx] = read_k(sK0, idx);
+#pragma unroll
+      for (int idx = 0; idx < 16; ++idx) {
+        const int t = idx >> 3, kk = idx & 7;
+        sA[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kbuf[idx % PD], qf[kk], kk == 0 ? zero16 : sA[t], 0, 0, 0);
+        if (idx + PD < 16) kbuf[idx % PD] = read_k(sK0, idx + PD);
+      }
+      // keys past the end of the range repeat the last valid row (the loader clamps), so the max needs no mask
+      float mx = sA[0][0];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sA[t][v]);
+      m_new = half_swap_max(mx);
+      alpha = 0.f;
+    }
+
+    // between iterations (tile `it` of parity P): lazy rescale, tail mask, publish the next tiles
+    auto top = [&](int it, auto pc, f32x16 (&s_cur)[2]) {
+      constexpr int P = decltype(pc)::value;
+      const int k0 = ks + it * BN;
+      if (it > 0 && __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // some row of this wave saw a new maximum
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+      }
+      if (k0 + BN > ke) {  // ragged last tile: keys >= ke do not exist
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) {
+            const int key = k0 + 32 * t + 8 * (v >> 2) + 4 * g + (v & 3);
+            if (key >= ke) s_cur[t][v] = -__builtin_inff();
+          }
+      }
+      wait_vmcnt<0>();
+      __syncthreads();  // K(it+1) and V(it) landed; K slot P and V slot P^1 are free
+      if (it + 2 < n_tiles) issue_mat(k0 + 2 * BN, P ? sK1 : sK0, false);
+      if (it + 1 < n_tiles) issue_mat(k0 + BN, P ? sV0 : sV1, true);
+    };
+    constexpr int SM_OPS = 96;
+
+    // one pipelined iteration for a tile of parity P
+    auto step = [&](int it, auto pc, f32x16 (&s_cur)[2], f32x16 (&s_nxt)[2]) {
+      constexpr int P = decltype(pc)::value;
+      top(it, pc, s_cur);
+      if (!wave_on) return;
+      const unsigned char* Kn = P ? sK0 : sK1;
+      const unsigned char* Vt = P ? sV1 : sV0;
+      const float mc = m_new * c;
+      const float m_prev = m_new;  // running max including tile it
+
+      float psum = 0.f;
+      float mxa = 0.f, mxb = 0.f, m_nx = 0.f, al_nx = 1.f;
+      // softmax micro-ops of tile it: group j = elements (2j, 2j+1) of the 32 this lane holds, 6 ops per group
+      // (the packed probabilities of slab s overwrite the first four of the eight score registers they came
+      // from, so P needs no registers of its own)
+      auto sm_op = [&](auto nc) {
+        constexpr int n = decltype(nc)::value;
+        constexpr int j = n / 6, k = n % 6;
+        constexpr int t = j >> 3, v0 = 2 * (j & 7);
+        constexpr int pw = 8 * ((j >> 2) & 1) + (j & 3);  // register of s_cur[t] that receives packed pair j
+        if constexpr (k == 0) s_cur[t][v0] = fmaf(s_cur[t][v0], c, -mc);
+        if constexpr (k == 1) s_cur[t][v0 + 1] = fmaf(s_cur[t][v0 + 1], c, -mc);
+        if constexpr (k == 2) s_cur[t][v0] = __builtin_amdgcn_exp2f(s_cur[t][v0]);
+        if constexpr (k == 3) s_cur[t][v0 + 1] = __builtin_amdgcn_exp2f(s_cur[t][v0 + 1]);
+        if constexpr (k == 4) s_cur[t][pw] = __builtin_bit_cast(float, pack_bf16x2(s_cur[t][v0], s_cur[t][v0 + 1]));
+        if constexpr (k == 5) {
+          const float packed = s_cur[t][pw];  // (a bit_cast applied to the vector element itself reads element 0)
+          psum = pair_sum(__builtin_bit_cast(unsigned, packed), psum);
+        }
+      };
+      auto p_operand = [&](int sl) -> bf16x8 {  // B operand of the PV MFMAs for slab sl
+        const f32x16& sv = s_cur[sl >> 1];
+        const f32x4 r = (sl & 1) ? __builtin_shufflevector(sv, sv, 8, 9, 10, 11) : __builtin_shufflevector(sv, sv, 0, 1, 2, 3);
+        return __builtin_bit_cast(bf16x8, r);
+      };
+      // row-max micro-ops of tile it+1: 8 + 8 max3, then combine / running max / alpha
+      auto mr_op = [&](auto nc) {
+        constexpr int n = decltype(nc)::value;
+        constexpr int q = n & 7;
+        if constexpr (n < 16) {
+          const f32x16& sv = s_nxt[n >> 3];
+          float& m = (n < 8) ? mxa : mxb;
+          if constexpr (q == 0) m = max3(sv[0], sv[1], sv[2]);
+          else if constexpr (q < 7) m = max3(m, sv[2 * q + 1], sv[2 * q + 2]);
+          else m = max3(m, sv[15], sv[15]);
+        } else if constexpr (n == 16) {
+          m_nx = half_swap_max(max3(mxa, mxb, mxb));
+        } else if constexpr (n == 17) {
+          m_nx = max3(m_prev, m_nx, m_nx);
+        } else if constexpr (n == 18) {
+          al_nx = __builtin_amdgcn_exp2f((m_prev - m_nx) * c);
+        }
+      };
+      bf16x8 obuf[PD];  // operand ring: K operands during the score MFMAs, then V operands
+#pragma unroll
+      for (int idx = 0; idx < PD; ++idx) obuf[idx] = read_k(Kn, idx);
+      // VALU work that does not wait for the operand reads
+      static_for<0, 6>(sm_op);
+      __builtin_amdgcn_sched_barrier(0);
+      static_for<0, 32>([&](auto chc) {
+        constexpr int ch = decltype(chc)::value;
+        if constexpr (ch < 16) {
+          constexpr int t = ch >> 3, kk = ch & 7;
+          s_nxt[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(obuf[ch % PD], qf[kk], kk == 0 ? zero16 : s_nxt[t], 0, 0, 0);
+          if constexpr (ch + PD < 16)
+            obuf[ch % PD] = read_k(Kn, ch + PD);
+          else
+            obuf[ch % PD] = read_v(Vt, ch + PD - 16);
+        } else {
+          constexpr int p = ch - 16;
+          o_acc[p & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(obuf[ch % PD], p_operand(p >> 2), o_acc[p & 3], 0, 0, 0);
+          if constexpr (p + PD < 16) obuf[ch % PD] = read_v(Vt, p + PD);
+        }
+        // softmax ops: all 96 done after chunk 25 (slab 3 is needed by chunk 28)
+        constexpr int lo = 6 + (90 * ch) / 26, hi0 = 6 + (90 * (ch + 1)) / 26, hi = hi0 < SM_OPS ? hi0 : SM_OPS;
+        static_for<(lo < hi ? lo : hi), hi>(sm_op);
+        // row max of tile it+1: first half of the scores is complete after chunk 7, the second after chunk 15
+        if constexpr (ch >= 10 && ch < 18) mr_op(std::integral_constant<int, ch - 10>{});
+        if constexpr (ch >= 19 && ch < 27) mr_op(std::integral_constant<int, ch - 19 + 8>{});
+        if constexpr (ch >= 28 && ch < 31) mr_op(std::integral_constant<int, ch - 28 + 16>{});
+        __builtin_amdgcn_sched_barrier(0);
+      });
+      l_run = l_run * alpha + psum;
+      m_run = m_prev;
+      m_new = m_nx;
+      alpha = al_nx;
+    };
+    // The last tile runs the same step: its score MFMAs read a K slot that holds no new tile and produce
+    // values nobody uses (one wasted product per workgroup instead of a second copy of the loop body).
+    const std::integral_constant<int, 0> even;
+    const std::integral_constant<int, 1> odd;
+    for (int it = 0; it < n_tiles; it += 2) {
+      step(it, even, sA, sB);
+      if (it + 1 >= n_tiles) break;
+      step(it + 1, odd, sB, sA);
+    }
+  } else {
   if (VSINGLE) {
     issue_mat(ks, &smem[0][0], false);
   } else {
@@ -301,17 +517,17 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
         }
     }
     // online softmax: every value this lane holds belongs to query i
-    float mx = s_acc[0][0];
+    float mx = max3(s_acc[0][0], s_acc[0][1], s_acc[0][2]);
 #pragma unroll
     for (int t = 0; t < NT; ++t)
 #pragma unroll
-      for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[t][v]);
-    mx = fmaxf(mx, __shfl_xor(mx, 32));
+      for (int v = (t == 0 ? 3 : 0); v < 16; v += 2) mx = max3(mx, s_acc[t][v], s_acc[t][v + 1 < 16 ? v + 1 : v]);
+    mx = half_swap_max(mx);
     const float m_new = fmaxf(m_run, mx);
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
     const float mc = m_new * c;
     m_run = m_new;
-    float psum = 0.f;
+    float psum = 0.f;  // row sum of the probabilities as rounded to bf16, i.e. of what the PV product uses
     bf16x8 pb[NS];
 #pragma unroll
     for (int s = 0; s < NS; ++s) {
@@ -320,8 +536,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       for (int e = 0; e < 8; e += 2) {
         const float p0 = __builtin_amdgcn_exp2f(s_acc[s >> 1][8 * (s & 1) + e] * c - mc);
         const float p1 = __builtin_amdgcn_exp2f(s_acc[s >> 1][8 * (s & 1) + e + 1] * c - mc);
-        psum += p0 + p1;
         pk[e >> 1] = pack_bf16x2(p0, p1);
+        psum = pair_sum(pk[e >> 1], psum);
       }
       pb[s] = __builtin_bit_cast(bf16x8, pk);
     }
@@ -351,6 +567,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       if (p + DV < RV) vbuf[p % DV] = read_v(p + DV);
     }
   }
+  }  // !PIPE
 
   if (!wave_on) return;
   // ---- epilogue: normalise and store ----
@@ -377,12 +594,16 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  if (a.block_m == 256)  // 8 waves, 256 query rows, 2 waves / SIMD
+  if (a.block_m == 256 && a.variant == 3)  // software-pipelined loop, 8 waves, 256 query rows, 2 waves / SIMD
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false, true>), dim3(grid), dim3(512), 0, stream, a);
+  else if (a.block_m == 256)  // 8 waves, 256 query rows, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false>), dim3(grid), dim3(512), 0, stream, a);
   else if (a.variant == 1)  // 32-key tiles, 3-stage ring, 3 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 32, 3, 3, false>), dim3(grid), dim3(256), 0, stream, a);
   else if (a.variant == 2)  // 64-key tiles, double-buffered K and V, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false>), dim3(grid), dim3(256), 0, stream, a);
+  else if (a.variant == 3)  // software-pipelined loop, 2 waves / SIMD
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false, true>), dim3(grid), dim3(256), 0, stream, a);
   else  // default: 64-key tiles, double-buffered K, single V slot, 3 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();

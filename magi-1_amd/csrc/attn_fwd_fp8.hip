@@ -152,8 +152,30 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
     if (k0 < k_split) pe = min(pe, k_split);
     return pe;
   };
+  const unsigned kvoff = (unsigned)row_in_tile0 * (unsigned)ks_t + (unsigned)(kchunk * 16);
+  const unsigned vvoff = (unsigned)row_in_tile0 * (unsigned)vs_t + (unsigned)(vchunk * 16);
+  const bool small_strides = ks_t * (BN + 8) < (1l << 31) && vs_t * (BN + 8) < (1l << 31);
+  const char* const kcol_u = a.k + (long)kvh * a.ks_h;  // wave-uniform column bases
+  const char* const vcol_u = a.v + (long)kvh * a.vs_h;
   auto issue_tile = [&](int k0, int pe, int buf) {
     const bool second = k0 >= k_split;
+    if (small_strides && k0 + BN <= pe) {
+      // full tile inside one piece: buffer-addressed direct loads (scalar base in the descriptor, one
+      // loop-invariant 32-bit lane offset, the row group in the scalar offset) cost the SIMD next to nothing
+      // to issue, unlike the same load with a 64-bit address per lane
+      const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc(
+          (void*)(kcol_u + (long)k0 * ks_t + (second ? k2_delta : 0)), 0, 0x7fffffff, 0x00020000);
+      const __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc(
+          (void*)(vcol_u + (long)k0 * vs_t + (second ? v2_delta : 0)), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+      for (int j = 0; j < LOADS; ++j) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, LDS_PTR(void, &smem[buf][0][(w + j * NW) * 1024]), 16, kvoff,
+                                                 (int)((unsigned)(8 * NW * j) * (unsigned)ks_t), 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, LDS_PTR(void, &smem[buf][1][(w + j * NW) * 1024]), 16, vvoff,
+                                                 (int)((unsigned)(8 * NW * j) * (unsigned)vs_t), 0, 0);
+      }
+      return;
+    }
     const char* kb = kcolp + (second ? k2_delta : 0);
     const char* vb = vcolp + (second ? v2_delta : 0);
 #pragma unroll

@@ -72,6 +72,11 @@ const char* magi_last_error(void);
  *                        "attend to the new KV without persisting it" (update_kv_cache == False,
  *                        dit_module.py:918-931) works without a copy.
  * out [total_q, Hq, D]   bf16, strides o_stride_t / o_stride_h
+ * out_group_heads, o_stride_g   optional two-level head addressing of `out` (0 = off): head h is written at
+ *                        (h / out_group_heads) * o_stride_g + (h % out_group_heads) * o_stride_h.  With 8 groups
+ *                        the core and the cross attention write straight into the "(hn n hd)" buffer that
+ *                        linear_proj consumes, which removes the concat + rearrange of attn_linear_proj
+ *                        (inference/model/dit/dit_module.py:1332-1340).
  * lse                    optional fp32 [Hq, total_q] (NULL to skip)
  * q_ranges, k_ranges     DEVICE int32 arrays, encoding per ranges_mode; clamped to
  *                        [0,total_q] / [0,total_k] in the kernel
@@ -105,6 +110,8 @@ typedef struct magi_attn_args {
   int32_t scale_chunk_tokens;
   float softmax_scale;
   int32_t flags; /* MAGI_ATTN_* bits */
+  int32_t out_group_heads;
+  int64_t o_stride_g;
 } magi_attn_args;
 
 int magi_attn_fwd(const magi_attn_args* args, void* stream);

@@ -62,6 +62,8 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     return fail(MAGI_EINVAL, "magi_attn_fwd: q/k/v/out must be 16-byte aligned");
   if (p->q_stride_h < p->D || p->k_stride_h < p->D || p->v_stride_h < p->D || p->o_stride_h < p->D)
     return fail(MAGI_EINVAL, "magi_attn_fwd: head stride smaller than head_dim");
+  if (p->out_group_heads < 0 || (p->out_group_heads > 0 && (p->Hq % p->out_group_heads || p->o_stride_g % 8)))
+    return fail(MAGI_EINVAL, "magi_attn_fwd: out_group_heads must divide Hq and o_stride_g keep rows 16-byte aligned");
   int k_split = p->total_k;
   if (p->k2 || p->v2) {
     if (!p->k2 || !p->v2) return fail(MAGI_EINVAL, "magi_attn_fwd: k2 and v2 must be given together");
@@ -96,6 +98,8 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.vs_h = p->v_stride_h * esz;
   a.os_t = p->o_stride_t * 2;
   a.os_h = p->o_stride_h * 2;
+  a.os_g = p->o_stride_g * 2;
+  a.out_group = p->out_group_heads;
   a.total_q = p->total_q;
   a.total_k = p->total_k;
   a.k_split = k_split;

@@ -136,6 +136,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   const unsigned tile = rem / (unsigned)a.G;
   const unsigned hg = rem - tile * (unsigned)a.G;
   const int h = (int)(kvh * a.G + hg);
+  // byte offset of this head in a row of `out` (optionally two-level: group, head in group)
+  const long o_head = a.out_group > 0 ? (long)(h / a.out_group) * a.os_g + (long)(h % a.out_group) * a.os_h : (long)h * a.os_h;
 
   // range with the rslot-th longest key span (ties by index)
   int ridx;
@@ -171,7 +173,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
   if (ke <= ks) {  // no keys: zeros, lse = -inf
     if (row_ok) {
-      char* op = a.out + (long)q_row * a.os_t + (long)h * a.os_h + g * 128;
+      char* op = a.out + (long)q_row * a.os_t + o_head + g * 128;
 #pragma unroll
       for (int c = 0; c < 8; ++c) *(u32x4*)(op + c * 16) = u32x4{0, 0, 0, 0};
       if (a.lse && g == 0) a.lse[(long)h * a.total_q + q_row] = -__builtin_inff();
@@ -574,7 +576,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.f / l_tot;
   if (row_ok) {
-    char* op = a.out + (long)q_row * a.os_t + (long)h * a.os_h;
+    char* op = a.out + (long)q_row * a.os_t + o_head;
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb)
 #pragma unroll

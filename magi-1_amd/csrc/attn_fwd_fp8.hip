@@ -72,6 +72,8 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   const unsigned tile = rem / (unsigned)a.G;
   const unsigned hg = rem - tile * (unsigned)a.G;
   const int h = (int)(kvh * a.G + hg);
+  // byte offset of this head in a row of `out` (optionally two-level: group, head in group)
+  const long o_head = a.out_group > 0 ? (long)(h / a.out_group) * a.os_g + (long)(h % a.out_group) * a.os_h : (long)h * a.os_h;
 
   int ridx;
   if (a.n_ranges <= MAX_SORT) {
@@ -106,7 +108,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
 
   if (ke <= ks) {
     if (row_ok) {
-      char* op = a.out + (long)q_row * a.os_t + (long)h * a.os_h + g * 128;
+      char* op = a.out + (long)q_row * a.os_t + o_head + g * 128;
 #pragma unroll
       for (int c = 0; c < 8; ++c) *(u32x4*)(op + c * 16) = u32x4{0, 0, 0, 0};
       if (a.lse && g == 0) a.lse[(long)h * a.total_q + q_row] = -__builtin_inff();
@@ -387,7 +389,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = v_max * __builtin_amdgcn_exp2f(-P_SHIFT) / l_tot;
   if (row_ok) {
-    char* op = a.out + (long)q_row * a.os_t + (long)h * a.os_h;
+    char* op = a.out + (long)q_row * a.os_t + o_head;
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb)
 #pragma unroll

@@ -20,6 +20,8 @@ struct AttnKernArgs {
   const float* k_scale;
   const float* v_scale;
   long qs_t, qs_h, ks_t, ks_h, vs_t, vs_h, os_t, os_h;
+  long os_g;     // byte stride between output head groups (out_group > 0)
+  int out_group; // heads per output group, 0 = heads addressed by os_h alone
   int total_q, total_k, k_split;
   int n_ranges, ranges_mode, tiles_per_range;
   int block_m;  // q rows per workgroup: 128 (4 waves) or 256 (8 waves)

@@ -42,6 +42,7 @@ class AttnArgs(C.Structure):
         ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32),
         ("dtype", C.c_int32), ("scale_chunk_tokens", C.c_int32),
         ("softmax_scale", C.c_float), ("flags", C.c_int32),
+        ("out_group_heads", C.c_int32), ("o_stride_g", C.c_int64),
     ]
 
 

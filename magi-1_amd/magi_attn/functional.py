@@ -117,7 +117,12 @@ def range_attention(
     a.q_stride_t, a.q_stride_h = q.stride(0), q.stride(1)
     a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1)
     a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1)
-    a.o_stride_t, a.o_stride_h = out.stride(0), out.stride(1)
+    if out.dim() == 4:  # [Tq, groups, heads per group, D]: two-level head addressing
+        if out.shape[0] != Tq or out.shape[1] * out.shape[2] != Hq or out.shape[3] != D or out.stride(3) != 1:
+            raise ValueError("a 4-D out must be [Tq, groups, Hq / groups, D] with contiguous rows")
+        a.o_stride_t, a.o_stride_g, a.o_stride_h, a.out_group_heads = out.stride(0), out.stride(1), out.stride(2), out.shape[2]
+    else:
+        a.o_stride_t, a.o_stride_h = out.stride(0), out.stride(1)
     a.total_q, a.total_k = Tq, total_k
     a.k_split = total_k if k2 is None else int(k_split)
     a.n_ranges, a.ranges_mode = max(n, 0), ranges_mode

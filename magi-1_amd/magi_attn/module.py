@@ -32,6 +32,18 @@ from .functional import head_norm, qk_prologue, range_attention
 from .params import InferenceParams, ModelMetaArgs, PackedCrossAttnParams
 
 
+PROJ_GROUPS = 8  # head groups of the linear_proj input (hard-coded "hn=8", dit_module.py:1338)
+
+
+def attn_linear_proj_input(core_attn_out: torch.Tensor, cross_attn_out: torch.Tensor) -> torch.Tensor:
+    """[sq, b, Hq*D] x 2 -> [sq, b, 2*Hq*D] in "(hn n hd)" order: the concat + rearrange that precedes linear_proj
+    in attn_linear_proj (dit_module.py:1336-1339), done with torch copies."""
+    sq, b, hd = core_attn_out.shape
+    both = torch.stack([core_attn_out.reshape(sq, b, PROJ_GROUPS, hd // PROJ_GROUPS),
+                        cross_attn_out.reshape(sq, b, PROJ_GROUPS, hd // PROJ_GROUPS)], dim=3)
+    return both.reshape(sq, b, 2 * hd)
+
+
 class FusedLayerNorm(torch.nn.Module):
     """Parameter holder of a per-head LayerNorm with zero-centred gamma (dit_module.py:323-357).
     The arithmetic runs inside the fused kernels; forward() is the stand-alone form."""
@@ -222,13 +234,14 @@ class FullyParallelAttention(torch.nn.Module):
         return key_and_value[..., :D].contiguous(), key_and_value[..., D:].contiguous()
 
     def core_attention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, bs: int,
-                       meta_args: ModelMetaArgs) -> torch.Tensor:
+                       meta_args: ModelMetaArgs, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         """query [(sq b), Hq, D], key / value [(sk b), Hkv, D] -> [(sq b), Hq, D]; dit_module.py:1023-1066.
-        bs > 1 only occurs with one range per batch row (asserted there too)."""
+        bs > 1 only occurs with one range per batch row (asserted there too).  `out` (bs == 1 only) is a
+        destination view, possibly in the grouped layout of range_attention."""
         p = meta_args.core_attn_params
         if bs == 1:
             out, _ = range_attention(query, key, value, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                     return_lse=False)
+                                     out=out, return_lse=False)
             return out
         if meta_args.denoising_range_num > 1:
             raise ValueError("bs > 1 with several denoising ranges is not a layout the pipeline produces")
@@ -242,20 +255,36 @@ class FullyParallelAttention(torch.nn.Module):
         return out
 
     def cross_attention(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor,
-                        cross_attn_params: PackedCrossAttnParams, get_xqkv_func: Callable) -> torch.Tensor:
-        """-> [sq, b, Hq*D]; dit_module.py:1098-1136."""
+                        cross_attn_params: PackedCrossAttnParams, get_xqkv_func: Callable,
+                        out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """-> [sq, b, Hq*D]; dit_module.py:1098-1136.  With `out` (b == 1 only: a destination view, possibly in
+        the grouped layout of range_attention) the result is written there (segments without text get zero rows
+        from the kernel) and `out` is returned."""
         qx, kx, vx = get_xqkv_func(mixed_qqkv, key_value_states)
-        out, _ = range_attention(qx, kx, vx, cross_attn_params.cu_seqlens_q, cross_attn_params.cu_seqlens_kv,
-                                 cross_attn_params.max_seqlen_q, cross_attn_params.max_seqlen_kv,
-                                 ranges_mode=L.MAGI_RANGES_CU, return_lse=False)
         b = mixed_qqkv.shape[1]
         sq = mixed_qqkv.shape[0]
+        if out is not None:
+            if b != 1:
+                raise ValueError("a destination view for the cross attention needs batch 1")
+            range_attention(qx, kx, vx, cross_attn_params.cu_seqlens_q, cross_attn_params.cu_seqlens_kv,
+                            cross_attn_params.max_seqlen_q, cross_attn_params.max_seqlen_kv,
+                            ranges_mode=L.MAGI_RANGES_CU, out=out, return_lse=False)
+            return out
+        out, _ = range_attention(qx, kx, vx, cross_attn_params.cu_seqlens_q, cross_attn_params.cu_seqlens_kv,
+                                 cross_attn_params.max_seqlen_q, cross_attn_params.max_seqlen_kv,
+                                 ranges_mode=L.MAGI_RANGES_CU, return_lse=False, zero_init=True)
         out = out.view(b, sq, -1)
         return out.transpose(0, 1).contiguous() if b > 1 else out.view(sq, 1, -1)
 
     # ------------------------------------------------------------------ forward
     def forward(self, hidden_states: torch.Tensor, key_value_states: torch.Tensor,
-                inference_params: Optional[InferenceParams], rotary_pos_emb: torch.Tensor, meta_args: ModelMetaArgs):
+                inference_params: Optional[InferenceParams], rotary_pos_emb: torch.Tensor, meta_args: ModelMetaArgs,
+                proj_layout: bool = False):
+        """-> (core_attn_out, xattn_out), each [sq, b, Hq*D], as the reference (dit_module.py:1138-1173).
+
+        With proj_layout=True the return value is ONE tensor [sq, b, 2*Hq*D] already in the "(hn n hd)" order
+        that linear_proj consumes (what attn_linear_proj builds with concat + rearrange, dit_module.py:1332-1340):
+        at batch 1 both attention launches write straight into it."""
         if rotary_pos_emb is None:
             raise ValueError("FullyParallelAttention needs rotary_pos_emb")
         sin_emb, cos_emb = rotary_pos_emb.tensor_split(2, -1)
@@ -264,12 +293,19 @@ class FullyParallelAttention(torch.nn.Module):
         D = self.hidden_size_per_attention_head
         mixed_qqkv = self.linear_qkv.forward_ln(hidden_states)
         p = meta_args.core_attn_params
+        Hq = self.num_attention_heads
+        fused = None
+        core_dst = cross_dst = None
+        if proj_layout and bs == 1 and Hq % PROJ_GROUPS == 0:
+            fused = torch.empty(sq, 1, 2 * Hq * D, dtype=hidden_states.dtype, device=hidden_states.device)
+            grouped = fused.view(sq, PROJ_GROUPS, 2, Hq // PROJ_GROUPS, D)
+            core_dst, cross_dst = grouped[:, :, 0], grouped[:, :, 1]
 
         use_cache = inference_params is not None and (
             meta_args.extract_prefix_video_feature or meta_args.fwd_extra_1st_chunk or meta_args.slice_point > 0)
         if not use_cache:
             q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb)
-            core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args)
+            core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst)
         else:
             if bs != 1 or inference_params.max_batch_size != 1:
                 raise ValueError("the cached path runs at batch 1 (as the reference pipeline does)")
@@ -291,10 +327,16 @@ class FullyParallelAttention(torch.nn.Module):
             kc, vc = cache[:split, :, :D], cache[:split, :, D:]
             if tail is None:
                 core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                          return_lse=False)
+                                          out=core_dst, return_lse=False)
             else:
                 core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                          k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, return_lse=False)
+                                          k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, out=core_dst,
+                                          return_lse=False)
+        if fused is not None:
+            self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, self.get_xqkv, out=cross_dst)
+            return fused
         core_attn_out = core.view(sq, bs, -1)
         xattn_out = self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, self.get_xqkv)
+        if proj_layout:
+            return attn_linear_proj_input(core_attn_out, xattn_out)
         return core_attn_out, xattn_out

@@ -289,6 +289,15 @@ def varlen_cross_attention(q, k, v, cu_seqlens_q, cu_seqlens_k, softmax_scale=No
     return range_attention(q, k, v, qr, kr, softmax_scale, dtype)
 
 
+def attn_linear_proj_input(core_attn_out: torch.Tensor, cross_attn_out: torch.Tensor, hn: int = 8) -> torch.Tensor:
+    """Input of linear_proj as attn_linear_proj builds it (dit_module.py:1336-1339):
+    cat([core, cross], dim=2) viewed "(n hn hd)" with n = 2 and re-ordered to "(hn n hd)".
+    core / cross [sq, b, Hq*D] -> [sq, b, 2*Hq*D]."""
+    sq, b, width = core_attn_out.shape
+    cat = torch.cat([core_attn_out, cross_attn_out], dim=2)      # (n hn hd)
+    return cat.view(sq, b, 2, hn, width // hn).permute(0, 1, 3, 2, 4).reshape(sq, b, 2 * width)
+
+
 def cross_attn_params_from_mask(xattn_mask: torch.Tensor, clip_token_nums: int):
     """cu_seqlens / ranges as dit_model.py:213-241 builds them.  xattn_mask [n_seg, L] of 0/1."""
     y_index = xattn_mask.reshape(xattn_mask.shape[0], -1).sum(-1).to(torch.int64)

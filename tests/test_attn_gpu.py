@@ -233,3 +233,21 @@ def test_full_size_480p_layer(dev):
 
 def test_full_size_720p_layer(dev):
     _full_size_check(dev, 21600, 4, 8, 48, 8, seed=3234, rows_per_chunk=128, cpu_rows=4)
+
+
+def test_grouped_output_layout(dev):
+    # out as [Tq, groups, heads per group, D] inside a wider buffer: same values as the plain layout, bit for bit,
+    # and nothing written outside the destination
+    L, sp, dn, Hq, Hkv = 77, 1, 2, 12, 4
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=21)
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    tq, tk = _ranges(dev, qr, kr)
+    plain, _ = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L)
+    for groups in (4, 2, 12):
+        buf = torch.full((dn * L, groups, 2, Hq // groups, 128), 7.0, dtype=torch.bfloat16, device=dev)
+        M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, out=buf[:, :, 1], return_lse=False)
+        assert torch.equal(buf[:, :, 1].reshape(dn * L, Hq, 128), plain)
+        assert torch.all(buf[:, :, 0] == 7.0)
+    with pytest.raises(ValueError):
+        M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L,
+                          out=torch.empty(dn * L, 5, 2, 128, dtype=torch.bfloat16, device=dev))

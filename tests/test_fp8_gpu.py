@@ -166,3 +166,20 @@ def test_fp8_full_size_720p_speedup_and_accuracy(dev):
             ref[:, hk * G:(hk + 1) * G] = torch.einsum("rgk,kd->rgd", torch.softmax(s, -1), v[:ke, hk].float())
         err, cos = _per_head(out[rows], ref)
         assert err <= 1e-2 and cos >= 0.998, (i, err, cos)
+
+
+def test_fp8_grouped_output_layout(dev):
+    # the fp8 kernel's epilogue honours the two-level head addressing of `out` like the bf16 one
+    L, dn, sp, Hq, Hkv, C = 90, 2, 1, 8, 2, 90
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=77)
+    q8, qs = M.quantize_fp8(q.to(dev), C)
+    k8, ks = M.quantize_fp8(k.to(dev), C)
+    v8, vs = M.quantize_fp8(v.to(dev), C)
+    tq = torch.tensor(O.q_ranges_for(dn, L), device=dev)
+    tk = torch.tensor(O.default_kvrange(sp, dn, L), device=dev)
+    kw = dict(q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=C, return_lse=False)
+    plain, _ = M.range_attention(q8, k8, v8, tq, tk, L, **kw)
+    buf = torch.full((dn * L, 4, 2, Hq // 4, 128), 3.0, dtype=torch.bfloat16, device=dev)
+    M.range_attention(q8, k8, v8, tq, tk, L, out=buf[:, :, 0], **kw)
+    assert torch.equal(buf[:, :, 0].reshape(dn * L, Hq, 128), plain)
+    assert torch.all(buf[:, :, 1] == 3.0)

@@ -286,6 +286,22 @@ def test_kv_cache_model_against_list_of_chunks():
                 assert torch.equal(cache.mem[c * L:(c + 1) * L], chunks[c])
 
 
+def test_attn_linear_proj_input_index_by_index():
+    # (n hn hd) -> (hn n hd) with n = 2, hn = 8, checked element by element against the index formula
+    sq, b, Hq, D = 3, 2, 16, 4
+    core = torch.arange(sq * b * Hq * D, dtype=torch.float32).view(sq, b, Hq * D)
+    cross = -core - 1
+    got = O.attn_linear_proj_input(core, cross)
+    assert got.shape == (sq, b, 2 * Hq * D)
+    hd = Hq * D // 8
+    for s_ in range(sq):
+        for b_ in range(b):
+            for hn in range(8):
+                for n, src in ((0, core), (1, cross)):
+                    for d in range(hd):
+                        assert got[s_, b_, hn * 2 * hd + n * hd + d] == src[s_, b_, hn * hd + d]
+
+
 # ----------------------------------------------------------------------------- chunk-window arithmetic
 def test_generate_sequences_reference_comment_examples():
     # the four worked examples kept next to the function in the reference (video_generate.py:139-161),

@@ -230,3 +230,55 @@ def test_layer_batched_cacheless_pass(dev):
                                      torch.tensor([0, L]), torch.tensor([0, int(lens[b])]), has_ip=False)
         assert (core[:, b].float().cpu() - c_ref[:, 0].float()).abs().max() <= 3e-2
         assert (xo[:, b].float().cpu() - x_ref[:, 0].float()).abs().max() <= 3e-2
+
+
+def test_layer_output_in_linear_proj_layout(dev):
+    """proj_layout=True: both attention launches write into the "(hn n hd)" buffer that linear_proj consumes
+    (dit_module.py:1336-1339).  Same kernels, other store addresses: bit-identical to re-ordering the two
+    separate outputs, with and without the KV cache, and through the torch fallback at batch > 1."""
+    hidden, Hq, Hkv, D = 256, 16, 8, 128
+    fr, H, W = 1, 3, 5
+    L = fr * H * W
+    layer = _make_layer(dev, hidden, Hq, Hkv, seed=5)
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+    rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
+    g = torch.Generator().manual_seed(6)
+    ip = P.InferenceParams(1, 4 * L)
+    ip.update_kv_cache = True
+    for sp, dn, has_ip in ((0, 2, True), (2, 2, True), (0, 2, False)):
+        S = dn * L
+        hs = torch.randn(S, 1, hidden, generator=g).bfloat16().to(dev)
+        lens = torch.tensor([5, 0][:dn])
+        mask = (torch.arange(8)[None] < lens[:, None]).float().view(dn, 1, 1, 8)
+        y = (torch.randn(int(lens.sum()), hidden, generator=g) * 0.5).bfloat16().to(dev)
+        k_range = R.generate_default_kvrange(sp, dn, L) if has_ip else R.generate_kv_range_for_uncondition(dn, L)
+        meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=sp, denoising_range_num=dn,
+                               range_num=sp + dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=True,
+                               distill_nearly_clean_chunk=False, clip_token_nums=L, enable_cuda_graph=False,
+                               core_attn_params=P.build_core_attn_params(R.q_ranges_from_chunks(dn, L).to(dev),
+                                                                         k_range.to(dev), L),
+                               cross_attn_params=P.build_cross_attn_params(mask.to(dev), L, 8))
+        rope = rope_mod.get_embed_for_forward(dn * fr, H, W, sp, dn)
+        with torch.no_grad():
+            core, xo = layer(hs, y, ip if has_ip else None, rope, meta)
+            fused = layer(hs, y, ip if has_ip else None, rope, meta, proj_layout=True)
+        assert fused.shape == (S, 1, 2 * Hq * D)
+        assert torch.equal(fused.cpu(), O.attn_linear_proj_input(core.cpu(), xo.cpu()))
+        assert torch.count_nonzero(xo[L:]).item() == 0  # the chunk without text
+    # batch > 1: no single-stride destination exists, the module re-orders with torch
+    B = 2
+    hs = torch.randn(L, B, hidden, generator=g).bfloat16().to(dev)
+    lens = torch.tensor([4, 8])
+    mask = (torch.arange(8)[None] < lens[:, None]).float().view(B, 1, 1, 8)
+    y = (torch.randn(int(lens.sum()), hidden, generator=g) * 0.5).bfloat16().to(dev)
+    kr = R.generate_kv_range_for_uncondition(B, L)
+    meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=0, denoising_range_num=1,
+                           range_num=1, extract_prefix_video_feature=False, fwd_extra_1st_chunk=False,
+                           distill_nearly_clean_chunk=False, clip_token_nums=L, enable_cuda_graph=False,
+                           core_attn_params=P.build_core_attn_params(kr.to(dev), kr.to(dev), L),
+                           cross_attn_params=P.build_cross_attn_params(mask.to(dev), L, 8))
+    rope = rope_mod.get_embed_for_forward(fr, H, W, 0, 1)
+    with torch.no_grad():
+        core, xo = layer(hs, y, None, rope, meta)
+        fused = layer(hs, y, None, rope, meta, proj_layout=True)
+    assert torch.equal(fused.cpu(), O.attn_linear_proj_input(core.cpu(), xo.cpu()))

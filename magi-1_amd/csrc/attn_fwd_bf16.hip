@@ -29,6 +29,7 @@
 // same keys at about the same time (each XCD has its own L2).  Ranges are visited longest
 // first.  Fully masked key tiles never exist: a rectangle is walked from k_start to k_end only.
 #include "kernels.h"
+#include "wave_ops.h"
 
 #include <type_traits>
 
@@ -83,19 +84,6 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
   asm volatile("" ::: "memory");
-}
-
-// wave-wide max of the two half-waves' values (lane i and lane i + 32 hold the same query)
-__device__ __forceinline__ float half_swap_max(float x) {
-  const unsigned u = __builtin_bit_cast(unsigned, x);
-  const u32x2 r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-  return fmaxf(__builtin_bit_cast(float, r[0]), __builtin_bit_cast(float, r[1]));
-}
-
-__device__ __forceinline__ float max3(float a, float b, float c) {
-  float r;
-  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
-  return r;
 }
 
 // p0 + p1 + acc for a packed pair of bf16 values

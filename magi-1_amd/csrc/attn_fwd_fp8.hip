@@ -11,6 +11,7 @@
 //     the softmax scale, the V scale (relative to the largest V scale of the range) joins the exp2
 //     exponent, and the Q scale is a per-lane constant because a lane owns one query.
 #include "kernels.h"
+#include "wave_ops.h"
 
 namespace magi {
 namespace {
@@ -303,12 +304,12 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
             if (key >= pe) s_acc[t][v] = -__builtin_inff();
           }
       }
-      float mx = s_acc[0][0];
+      float mx = max3(s_acc[0][0], s_acc[0][1], s_acc[0][2]);
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, s_acc[t][v]);
-      mx = fmaxf(mx, __shfl_xor(mx, 32));
+        for (int v = (t == 0 ? 3 : 0); v < 16; v += 2) mx = max3(mx, s_acc[t][v], s_acc[t][v + 1 < 16 ? v + 1 : v]);
+      mx = half_swap_max(mx);
       if constexpr (POW2) {
         // s_acc already holds exponent - m_run + shift; a value above `shift` is a new row maximum
         const float over = mx - shift;

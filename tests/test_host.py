@@ -75,6 +75,11 @@ def test_attn_argument_validation_without_gpu():
     a.q_stride_h = a.o_stride_h = 128
     a.k_stride_t, a.k_stride_h, a.v_stride_t, a.v_stride_h = 256, 128, 256, 100
     assert lib.magi_attn_fwd(C.byref(a), None) == -22  # misaligned stride
+    a.v_stride_h = 128
+    a.k = a.v = 4096
+    a.total_k = 8
+    a.out_group_heads = 3  # does not divide Hq = 4
+    assert lib.magi_attn_fwd(C.byref(a), None) == -22 and b"out_group_heads" in lib.magi_last_error()
     assert lib.magi_attn_fwd(None, None) == -22
 
 

@@ -213,7 +213,13 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * NW * 1024), 16, voff,
                                                  (int)((unsigned)(4 * NW * j) * (unsigned)st), 0, 0);
     } else {  // ragged end of the range, or a tile that straddles the two key segments
-      const int chunk = is_v ? vchunk : kchunk;
+      // (rare: the lane geometry is re-derived here from an opaque copy of the lane index, so that nothing of
+      // it occupies registers across the main loop)
+      int lane = l;
+      asm volatile("" : "+v"(lane));
+      const int lrow_s = lane >> 4, slot_s = lane & 15;
+      const int row_in_tile0 = 4 * w + lrow_s;
+      const int chunk = is_v ? (slot_s ^ (lrow_s << 2)) : (slot_s ^ ((4 * (w & 3) + lrow_s) & 15));
 #pragma unroll
       for (int j = 0; j < LOADS; ++j) {
         const int row = min(k0 + row_in_tile0 + 4 * NW * j, ke - 1);
@@ -518,19 +524,19 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
     const float mc = m_new * c;
     m_run = m_new;
     float psum = 0.f;  // row sum of the probabilities as rounded to bf16, i.e. of what the PV product uses
-    bf16x8 pb[NS];
+    // the packed probabilities of slab s overwrite the first four of the eight score registers they came from
 #pragma unroll
-    for (int s = 0; s < NS; ++s) {
-      u32x4 pk;
+    for (int s = 0; s < NS; ++s)
 #pragma unroll
       for (int e = 0; e < 8; e += 2) {
-        const float p0 = __builtin_amdgcn_exp2f(s_acc[s >> 1][8 * (s & 1) + e] * c - mc);
-        const float p1 = __builtin_amdgcn_exp2f(s_acc[s >> 1][8 * (s & 1) + e + 1] * c - mc);
-        pk[e >> 1] = pack_bf16x2(p0, p1);
-        psum = pair_sum(pk[e >> 1], psum);
+        f32x16& sv = s_acc[s >> 1];
+        const int v0 = 8 * (s & 1) + e;
+        const float p0 = __builtin_amdgcn_exp2f(sv[v0] * c - mc);
+        const float p1 = __builtin_amdgcn_exp2f(sv[v0 + 1] * c - mc);
+        const unsigned pk = pack_bf16x2(p0, p1);
+        psum = pair_sum(pk, psum);
+        sv[8 * (s & 1) + (e >> 1)] = __builtin_bit_cast(float, pk);
       }
-      pb[s] = __builtin_bit_cast(bf16x8, pk);
-    }
     l_run = l_run * alpha + psum;
     if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // some row of this wave saw a new maximum
 #pragma unroll
@@ -538,6 +544,11 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 #pragma unroll
         for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
     }
+    auto p_operand = [&](int s) -> bf16x8 {  // B operand of the PV MFMAs for slab s
+      const f32x16& sv = s_acc[s >> 1];
+      const f32x4 r = (s & 1) ? __builtin_shufflevector(sv, sv, 8, 9, 10, 11) : __builtin_shufflevector(sv, sv, 0, 1, 2, 3);
+      return __builtin_bit_cast(bf16x8, r);
+    };
 
     // O^T[d][q] += V^T[d][key] P^T[key][q]; V operands run DV reads ahead
     __builtin_amdgcn_sched_barrier(0);
@@ -553,7 +564,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 #pragma unroll
     for (int p = 0; p < RV; ++p) {
       const int mb = p / NS, s = p % NS;
-      o_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vbuf[p % DV], pb[s], o_acc[mb], 0, 0, 0);
+      o_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vbuf[p % DV], p_operand(s), o_acc[mb], 0, 0, 0);
       if (p + DV < RV) vbuf[p % DV] = read_v(p + DV);
     }
   }

@@ -51,7 +51,7 @@ def test_chunk_causal_parity(dev, L, dn, sp, Hq, Hkv):
     out, lse = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, int(kr.max() - kr.min()))
     assert out.dtype == torch.bfloat16 and out.shape == q.shape and lse.shape == (Hq, dn * L)
     _cmp(out, ref, f"L={L}")
-    # Q is pre-multiplied by scale * log2(e) and re-rounded to bf16 once per workgroup: ~1e-3 on the logits
+    # the kernel's row sum runs over the probabilities as rounded to bf16 (what the PV product uses): ~1e-3
     assert (lse.cpu() - lse_ref).abs().max() < 5e-3
 
 
@@ -251,3 +251,23 @@ def test_grouped_output_layout(dev):
     with pytest.raises(ValueError):
         M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L,
                           out=torch.empty(dn * L, 5, 2, 128, dtype=torch.bfloat16, device=dev))
+
+
+def test_more_ranges_than_the_in_kernel_ranking_handles(dev):
+    # above 256 ranges the kernel skips the longest-first ranking and maps range slots in reverse index order;
+    # results must not depend on it (cu_seqlens form: 300 segments, some of them without keys)
+    rng = np.random.default_rng(3)
+    n = 300
+    ql = rng.integers(1, 40, size=n)
+    kl = rng.integers(0, 70, size=n)
+    kl[::17] = 0
+    cu_q = np.concatenate([[0], np.cumsum(ql)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(kl)]).astype(np.int32)
+    Hq, Hkv = 4, 2
+    q, k, v = O.synthetic_qkv(int(cu_q[-1]), int(cu_k[-1]), Hq, Hkv, 128, seed=31)
+    ref = O.varlen_cross_attention(q, k, v, cu_q, cu_k)
+    out = M.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), torch.tensor(cu_q, device=dev),
+                                   torch.tensor(cu_k, device=dev), int(ql.max()), int(kl.max()))
+    _cmp(out, ref, "300 segments")
+    empty_rows = np.concatenate([np.arange(cu_q[i], cu_q[i + 1]) for i in range(n) if kl[i] == 0])
+    assert torch.count_nonzero(out[torch.tensor(empty_rows, device=dev)]).item() == 0

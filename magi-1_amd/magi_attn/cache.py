@@ -1,0 +1,60 @@
+"""One HBM arena for the KV caches of all layers.
+
+The reference allocates each layer's cache lazily on first use (`_allocate_key_and_value_memory`,
+inference/model/dit/dit_module.py:800-819, keyed by layer number in
+`InferenceParams.key_value_memory_dict`, :905-912) and ships `kv_offload: true` for the 24B model
+(example/24B/24B_base_config.json:83), which keeps the caches in pinned host memory and copies the prefix to the
+GPU in every layer (:915).  A 720p 24B generation needs 48 layers x 1.06 GB = 51 GB; an MI355X has 288 GB, so the
+caches stay resident: one allocation made up front, one view per layer, no host staging, no allocator traffic
+inside the denoising loop.  The attention kernels read the views in place."""
+from __future__ import annotations
+
+from typing import Dict, Iterable, Optional
+
+import torch
+
+from .params import InferenceParams
+
+
+class KVCacheArena:
+    """[num_layers, max_sequence_length * max_batch_size, Hkv, 2*D]; layer i's cache is `arena[i]`, K in
+    [..., :D] and V in [..., D:], the layout of the reference's per-layer tensor."""
+
+    def __init__(self, num_layers: int, max_sequence_length: int, num_query_groups: int, head_dim: int = 128,
+                 max_batch_size: int = 1, dtype: torch.dtype = torch.bfloat16, device=None,
+                 memory_budget_bytes: Optional[int] = None, kv_offload: bool = False):
+        if kv_offload:
+            raise ValueError("kv_offload is not offered: the caches of every layer fit in HBM (see the module docstring)")
+        if min(num_layers, max_sequence_length, num_query_groups, head_dim, max_batch_size) <= 0:
+            raise ValueError("all sizes must be positive")
+        self.num_layers = num_layers
+        self.max_sequence_length = max_sequence_length
+        self.max_batch_size = max_batch_size
+        rows = max_sequence_length * max_batch_size
+        need = self.bytes_needed(num_layers, max_sequence_length, num_query_groups, head_dim, max_batch_size, dtype)
+        if memory_budget_bytes is not None and need > memory_budget_bytes:
+            raise MemoryError(f"KV caches need {need / 2**30:.1f} GiB, budget is {memory_budget_bytes / 2**30:.1f} GiB")
+        self.buffer = torch.empty(num_layers, rows, num_query_groups, 2 * head_dim, dtype=dtype, device=device)
+
+    @staticmethod
+    def bytes_needed(num_layers: int, max_sequence_length: int, num_query_groups: int, head_dim: int = 128,
+                     max_batch_size: int = 1, dtype: torch.dtype = torch.bfloat16) -> int:
+        return (num_layers * max_sequence_length * max_batch_size * num_query_groups * 2 * head_dim
+                * torch.empty((), dtype=dtype).element_size())
+
+    def layer(self, index: int) -> torch.Tensor:
+        return self.buffer[index]
+
+    def attach(self, inference_params: InferenceParams, layer_numbers: Optional[Iterable[int]] = None
+               ) -> Dict[int, torch.Tensor]:
+        """Hands the layer views to `inference_params.key_value_memory_dict` (what the attention module looks
+        up by layer number); `layer_numbers` defaults to 0 .. num_layers-1 in arena order."""
+        if (inference_params.max_sequence_length != self.max_sequence_length
+                or inference_params.max_batch_size != self.max_batch_size):
+            raise ValueError("arena and InferenceParams disagree on max_sequence_length / max_batch_size")
+        numbers = list(range(self.num_layers)) if layer_numbers is None else list(layer_numbers)
+        if len(numbers) != self.num_layers or len(set(numbers)) != len(numbers):
+            raise ValueError("need one distinct layer number per arena layer")
+        for i, n in enumerate(numbers):
+            inference_params.key_value_memory_dict[n] = self.buffer[i]
+        return inference_params.key_value_memory_dict

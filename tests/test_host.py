@@ -159,3 +159,24 @@ def test_functional_rejects_cpu_tensors():
     r = torch.zeros(1, 2, dtype=torch.int32)
     with pytest.raises(ValueError):
         magi_attn.range_attention(q, q, q, r, r, 4)
+
+
+def test_kv_cache_arena_views_accounting_and_errors():
+    from magi_attn.cache import KVCacheArena
+    # the 24B 720p figure of the design notes: 48 layers x 259200 tokens x 8 heads x 256 x 2 B = 51 GB
+    assert KVCacheArena.bytes_needed(48, 259200, 8) == 48 * 259200 * 8 * 256 * 2
+    arena = KVCacheArena(3, 40, 2, device="cpu")
+    ip = P.InferenceParams(1, 40)
+    d = arena.attach(ip, layer_numbers=[5, 6, 7])
+    assert sorted(d) == [5, 6, 7] and d[6].shape == (40, 2, 256)
+    d[6][3, 1, 200] = 2.5  # a view: writes land in the arena, layers do not overlap
+    assert arena.layer(1)[3, 1, 200] == 2.5 and arena.buffer.data_ptr() == d[5].data_ptr()
+    assert d[7].data_ptr() - d[6].data_ptr() == 40 * 2 * 256 * 2
+    with pytest.raises(ValueError):
+        arena.attach(P.InferenceParams(1, 41))
+    with pytest.raises(ValueError):
+        arena.attach(ip, layer_numbers=[1, 1, 2])
+    with pytest.raises(MemoryError):
+        KVCacheArena(48, 259200, 8, device="cpu", memory_budget_bytes=1 << 30)
+    with pytest.raises(ValueError):
+        KVCacheArena(1, 8, 1, device="cpu", kv_offload=True)

@@ -282,3 +282,44 @@ def test_layer_output_in_linear_proj_layout(dev):
         core, xo = layer(hs, y, None, rope, meta)
         fused = layer(hs, y, None, rope, meta, proj_layout=True)
     assert torch.equal(fused.cpu(), O.attn_linear_proj_input(core.cpu(), xo.cpu()))
+
+
+def test_layer_with_arena_backed_cache(dev):
+    """The same cached forward with the lazily allocated per-layer cache and with a view of the all-layer arena:
+    identical outputs and identical cache rows."""
+    from magi_attn.cache import KVCacheArena
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+    hidden, Hq, Hkv, D = 256, 6, 2, 128
+    fr, H, W = 1, 4, 4
+    L = fr * H * W
+    layer = _make_layer(dev, hidden, Hq, Hkv, seed=7)
+    rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
+    outs = []
+    for use_arena in (False, True):
+        ip = P.InferenceParams(1, 4 * L)
+        ip.update_kv_cache = True
+        if use_arena:
+            arena = KVCacheArena(5, 4 * L, Hkv, device=dev)
+            arena.buffer.fill_(float("nan"))
+            arena.attach(ip)  # the layer's number (3) selects arena row 3
+        g = torch.Generator().manual_seed(8)
+        res = []
+        for sp, dn in ((0, 2), (2, 2)):
+            S = dn * L
+            hs = torch.randn(S, 1, hidden, generator=g).bfloat16().to(dev)
+            mask = torch.ones(dn, 1, 1, 8)
+            y = (torch.randn(dn * 8, hidden, generator=g) * 0.5).bfloat16().to(dev)
+            meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=sp,
+                                   denoising_range_num=dn, range_num=sp + dn, extract_prefix_video_feature=False,
+                                   fwd_extra_1st_chunk=True, distill_nearly_clean_chunk=False, clip_token_nums=L,
+                                   enable_cuda_graph=False,
+                                   core_attn_params=P.build_core_attn_params(R.q_ranges_from_chunks(dn, L).to(dev),
+                                                                             R.generate_default_kvrange(sp, dn, L).to(dev), L),
+                                   cross_attn_params=P.build_cross_attn_params(mask.to(dev), L, 8))
+            with torch.no_grad():
+                res.append(layer(hs, y, ip, rope_mod.get_embed_for_forward(dn * fr, H, W, sp, dn), meta))
+        outs.append((res, ip.key_value_memory_dict[3].clone()))
+    for (c0, x0), (c1, x1) in zip(outs[0][0], outs[1][0]):
+        assert torch.equal(c0, c1) and torch.equal(x0, x1)
+    assert torch.equal(outs[0][1][: 4 * L], outs[1][1][: 4 * L])
+    assert torch.isnan(arena.layer(2)).all() and torch.isnan(arena.layer(4)).all()  # other layers untouched

@@ -271,3 +271,53 @@ def test_more_ranges_than_the_in_kernel_ranking_handles(dev):
     _cmp(out, ref, "300 segments")
     empty_rows = np.concatenate([np.arange(cu_q[i], cu_q[i + 1]) for i in range(n) if kl[i] == 0])
     assert torch.count_nonzero(out[torch.tensor(empty_rows, device=dev)]).item() == 0
+
+
+def test_randomised_shapes_ranges_strides_and_splits(dev):
+    """Seeded sweep over head counts, range geometry (arbitrary starts, overlaps between K ranges, gaps between
+    Q ranges), strided / interleaved K-V storage and key-axis splits, each compared with the oracle."""
+    rng = np.random.default_rng(2024)
+    for case in range(24):
+        Hkv = int(rng.choice([1, 2, 3, 4]))
+        G = int(rng.choice([1, 2, 3, 6]))
+        Hq = Hkv * G
+        n = int(rng.integers(1, 6))
+        ql = rng.integers(1, 260, size=n)
+        gaps = rng.integers(0, 20, size=n)
+        q_start = np.cumsum(gaps + np.concatenate([[0], ql[:-1]]))
+        qr = np.stack([q_start, q_start + ql], 1)
+        Tq = int(qr[-1, 1] + rng.integers(0, 10))
+        Tk = int(rng.integers(1, 700))
+        ks = rng.integers(0, Tk, size=n)
+        kr = np.stack([ks, np.minimum(Tk, ks + rng.integers(0, 400, size=n))], 1)
+        q, k, v = O.synthetic_qkv(Tq, Tk, Hq, Hkv, 128, seed=5000 + case)
+        ref = O.range_attention(q, k, v, qr, kr)
+        covered = np.zeros(Tq, bool)
+        for a, b in qr:
+            covered[a:b] = True
+        tq, tk = _ranges(dev, qr, kr)
+        layout = case % 3
+        if layout == 0:  # separate contiguous K and V
+            kd, vd = k.to(dev), v.to(dev)
+        elif layout == 1:  # interleaved cache [T, Hkv, 2D]
+            cache = torch.cat([k, v], -1).to(dev)
+            kd, vd = cache[..., :128], cache[..., 128:]
+        else:  # padded rows: token stride larger than Hkv * D
+            pad = torch.zeros(Tk, Hkv + 1, 128, dtype=torch.bfloat16, device=dev)
+            pad2 = torch.zeros_like(pad)
+            pad[:, :Hkv] = k.to(dev)
+            pad2[:, :Hkv] = v.to(dev)
+            kd, vd = pad[:, :Hkv], pad2[:, :Hkv]
+        kw = {}
+        if case % 4 == 3:  # key axis = [first split rows | side buffer]
+            split = int(rng.integers(0, Tk + 1))
+            kw = dict(k2=kd[split:], v2=vd[split:], k_split=split)  # same strides as the first segment
+            kd, vd = kd[:split], vd[:split]
+        out, lse = M.range_attention(q.to(dev), kd, vd, tq, tk, int(ql.max()), **kw)
+        cov = torch.tensor(covered, device=dev)
+        if torch.count_nonzero(ref).item() == 0:  # every range of this case is empty
+            assert torch.count_nonzero(out).item() == 0
+        else:
+            _cmp(out[cov], ref[torch.tensor(covered)], f"case {case}")
+        assert torch.count_nonzero(out[~cov]).item() == 0, f"case {case}: uncovered rows written"
+        assert torch.isfinite(out).all()

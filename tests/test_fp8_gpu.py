@@ -183,3 +183,45 @@ def test_fp8_grouped_output_layout(dev):
     M.range_attention(q8, k8, v8, tq, tk, L, out=buf[:, :, 0], **kw)
     assert torch.equal(buf[:, :, 0].reshape(dn * L, Hq, 128), plain)
     assert torch.all(buf[:, :, 1] == 3.0)
+
+
+def test_fp8_randomised_ranges_chunks_and_splits(dev):
+    """Seeded sweep over head counts, range geometry, scale-chunk sizes (pieces of the key axis end at chunk
+    boundaries) and key-axis splits, in both scale modes, against the oracle on the dequantised inputs."""
+    import math
+    rng = np.random.default_rng(77)
+    cs = 128 ** -0.5 * math.log2(math.e)
+    for case in range(12):
+        Hkv = int(rng.choice([1, 2, 4]))
+        Hq = Hkv * int(rng.choice([1, 3, 6]))
+        n = int(rng.integers(1, 5))
+        ql = rng.integers(1, 200, size=n)
+        q_start = np.concatenate([[0], np.cumsum(ql[:-1])])
+        qr = np.stack([q_start, q_start + ql], 1)
+        Tq, Tk = int(ql.sum()), int(rng.integers(40, 600))
+        ks = rng.integers(0, Tk - 20, size=n)
+        kr = np.stack([ks, np.minimum(Tk, ks + rng.integers(1, 400, size=n))], 1)
+        C = int(rng.choice([32, 50, 64, 100, 1000]))
+        pow2 = case % 2 == 1
+        q, k, v = O.synthetic_qkv(Tq, Tk, Hq, Hkv, 128, seed=9000 + case)
+        v = (v.float() * (1 + 3 * (torch.arange(Tk) // C % 3))[:, None, None]).bfloat16()  # uneven V chunks
+        q8, qs = M.quantize_fp8(q.to(dev), C, premul=cs if pow2 else 1.0, pow2_scales=pow2)
+        k8, ksc = M.quantize_fp8(k.to(dev), C, pow2_scales=pow2)
+        v8, vsc = M.quantize_fp8(v.to(dev), C, pow2_scales=pow2)
+        tq = torch.tensor(qr, dtype=torch.int32, device=dev)
+        tk = torch.tensor(kr, dtype=torch.int32, device=dev)
+        kw = dict(q_scale=qs, k_scale=ksc, v_scale=vsc, scale_chunk_tokens=C, fp8_pow2_prescaled=pow2, return_lse=False)
+        k1, v1 = k8, v8
+        if case % 3 == 2:
+            split = int(rng.integers(0, Tk + 1))
+            kw.update(k2=k8[split:], v2=v8[split:], k_split=split)
+            k1, v1 = k8[:split], v8[:split]
+        out, _ = M.range_attention(q8, k1, v1, tq, tk, int(ql.max()), **kw)
+        qd = O.dequantize_per_head_chunk(q8.cpu(), qs.cpu(), C)
+        if pow2:
+            qd = qd / cs * 128 ** -0.5
+        ref = O.range_attention(qd, O.dequantize_per_head_chunk(k8.cpu(), ksc.cpu(), C),
+                                O.dequantize_per_head_chunk(v8.cpu(), vsc.cpu(), C), qr, kr, softmax_scale=1.0 if pow2 else None)
+        assert torch.isfinite(out).all(), f"case {case}"
+        rel = ((out.double().cpu() - ref.double()).abs().max() / ref.abs().max().clamp_min(1e-6)).item()
+        assert rel <= 4e-2, f"case {case}: {rel}"

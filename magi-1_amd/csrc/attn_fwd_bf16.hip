@@ -22,7 +22,9 @@
 // in different phases.  The default instantiation runs 3 waves / SIMD: <= 168 VGPRs (shallow
 // operand prefetch) and 48 KB of LDS per workgroup (64-key tiles, K double buffered, ONE V slot that
 // is refilled under the score MFMAs and the softmax of the same tile).  Instantiations with 2 waves
-// / SIMD (deep prefetch, K and V double buffered) and with 32-key tiles are kept for comparison.
+// / SIMD (deep prefetch, K and V double buffered), with 32-key tiles, and a software-pipelined loop
+// (PIPE: score MFMAs of the next tile, softmax and PV MFMAs of the current one interleaved in one
+// basic block, 2 waves / SIMD) are kept for comparison; on the 720p layer none is faster.
 //
 // Work decomposition: blockIdx -> (kv head, range slot, q tile, q head within the GQA group),
 // laid out so that the workgroups an XCD receives (blockIdx % 8) share a KV head and walk the
@@ -106,7 +108,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");
   static_assert(!PIPE || (NSTAGE == 2 && BN == 64 && !VSINGLE), "pipelined loop: 64-key tiles, two K slots and two V slots");
   // ring of NSTAGE (K tile, V tile) pairs, or in single-V mode K slot 0, K slot 1, V slot
-  // (pipelined loop: K slots 0, 1 and V slots 2, 3)
+  // (the pipelined loop declares its four slots as separate objects instead and leaves this one a stub)
   __shared__ __attribute__((aligned(1024))) unsigned char smem[PIPE ? 1 : VSINGLE ? 3 : 2 * NSTAGE][PIPE ? 16 : TILE_BYTES];
   __shared__ int s_sel;
 

@@ -13,6 +13,8 @@
 #include "kernels.h"
 #include "wave_ops.h"
 
+#include <type_traits>
+
 namespace magi {
 namespace {
 
@@ -57,7 +59,14 @@ __device__ __forceinline__ void load_range(const int* r, int mode, int i, int to
 
 template <bool POW2>
 __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKernArgs a) {
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[2][2][TILE_BYTES];  // [buffer][K|V]
+  // Two (K tile, V tile) buffers as four separate objects that are only ever indexed statically: the compiler
+  // then knows that a read of one buffer cannot alias the direct-to-LDS loads in flight to the other and does
+  // not make it wait for them (with one array and a run-time buffer index every LDS read waited for vmcnt(0),
+  // i.e. for the tile that had just been requested).
+  __shared__ __attribute__((aligned(1024))) unsigned char sK0[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sV0[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sK1[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sV1[TILE_BYTES];
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -150,8 +159,8 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   const char* const vcolp = a.v + (long)kvh * a.vs_h + vchunk * 16;
 
   // The key range is walked in pieces [k0, pe) that stay inside one scale chunk and one key segment.
-  auto piece_end = [&](int k0) {
-    int pe = min(ke, (k0 / C + 1) * C);
+  auto piece_end = [&](int k0, int chunk) {  // chunk = k0 / C
+    int pe = min(ke, (chunk + 1) * C);
     if (k0 < k_split) pe = min(pe, k_split);
     return pe;
   };
@@ -160,7 +169,10 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   const bool small_strides = ks_t * (BN + 8) < (1l << 31) && vs_t * (BN + 8) < (1l << 31);
   const char* const kcol_u = a.k + (long)kvh * a.ks_h;  // wave-uniform column bases
   const char* const vcol_u = a.v + (long)kvh * a.vs_h;
-  auto issue_tile = [&](int k0, int pe, int buf) {
+  auto issue_tile = [&](int k0, int pe, auto BUFC) {
+    constexpr int BUF = decltype(BUFC)::value;
+    unsigned char* const dK = BUF ? sK1 : sK0;
+    unsigned char* const dV = BUF ? sV1 : sV0;
     const bool second = k0 >= k_split;
     if (small_strides && k0 + BN <= pe) {
       // full tile inside one piece: buffer-addressed direct loads (scalar base in the descriptor, one
@@ -172,9 +184,9 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           (void*)(vcol_u + (long)k0 * vs_t + (second ? v2_delta : 0)), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
       for (int j = 0; j < LOADS; ++j) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, LDS_PTR(void, &smem[buf][0][(w + j * NW) * 1024]), 16, kvoff,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, LDS_PTR(void, dK + (w + j * NW) * 1024), 16, kvoff,
                                                  (int)((unsigned)(8 * NW * j) * (unsigned)ks_t), 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, LDS_PTR(void, &smem[buf][1][(w + j * NW) * 1024]), 16, vvoff,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, LDS_PTR(void, dV + (w + j * NW) * 1024), 16, vvoff,
                                                  (int)((unsigned)(8 * NW * j) * (unsigned)vs_t), 0, 0);
       }
       return;
@@ -184,9 +196,9 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
       const int row = min(k0 + row_in_tile0 + 8 * NW * j, pe - 1);
-      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kb + (long)row * ks_t), LDS_PTR(void, &smem[buf][0][(w + j * NW) * 1024]),
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kb + (long)row * ks_t), LDS_PTR(void, dK + (w + j * NW) * 1024),
                                        16, 0, 0);
-      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vb + (long)row * vs_t), LDS_PTR(void, &smem[buf][1][(w + j * NW) * 1024]),
+      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vb + (long)row * vs_t), LDS_PTR(void, dV + (w + j * NW) * 1024),
                                        16, 0, 0);
     }
   };
@@ -222,27 +234,42 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const float c_q = a.scale_log2 * q_sc;  // softmax scale * log2(e) * q scale
 
-  int k0 = ks, pe = piece_end(ks);
-  issue_tile(k0, pe, 0);
-  int buf = 0;
-  while (k0 < ke) {
-    int k1 = k0 + BN, pe1 = pe;  // the tile after this one
+  // Per-piece quantities, refreshed by the first tile of a piece: the scale loads (vector memory loads, whose
+  // wait would also wait for the tile just requested) and the divisions stay out of the steady-state loop.
+  // They are wave uniform and live in scalar registers.
+  int chunk = ks / C;
+  bool new_piece = true;
+  float c = 0.f, shift = 0.f, unshift = 0.f;
+  int e_k = 0;
+  int k0 = ks, pe = piece_end(ks, chunk);
+  issue_tile(k0, pe, std::integral_constant<int, 0>{});
+  auto tile_step = [&](auto BUFC) {
+    constexpr int BUF = decltype(BUFC)::value;
+    int k1 = k0 + BN, pe1 = pe, chunk1 = chunk;  // the tile after this one
+    bool new_piece1 = false;
     if (k1 >= pe) {
       k1 = pe;
-      pe1 = (k1 < ke) ? piece_end(k1) : ke;
+      chunk1 = chunk + (k1 == (chunk + 1) * C ? 1 : 0);
+      pe1 = (k1 < ke) ? piece_end(k1, chunk1) : ke;
+      new_piece1 = true;
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (k1 < ke) issue_tile(k1, pe1, buf ^ 1);
+    if (k1 < ke) issue_tile(k1, pe1, std::integral_constant<int, BUF ^ 1>{});
     if (wave_on) {
-      const unsigned char* Kt = &smem[buf][0][0];
-      const unsigned char* Vt = &smem[buf][1][0];
-      const int cidx = k0 / C;
-      const float k_sc = a.k_scale[(long)cidx * a.Hkv + kvh];
-      const float v_sc = a.v_scale[(long)cidx * a.Hkv + kvh];
-      const float c = c_q * k_sc;                                             // per-lane score scale of this tile
-      const float shift = P_SHIFT + __builtin_amdgcn_logf(v_sc) - log2_vmax;  // <= 8
-      const float unshift = __builtin_amdgcn_exp2f(-shift);
+      const unsigned char* const Kt = BUF ? sK1 : sK0;
+      const unsigned char* const Vt = BUF ? sV1 : sV0;
+      if (new_piece) {
+        auto uni = [](float x) {
+          return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
+        };
+        const float k_sc = uni(a.k_scale[(long)chunk * a.Hkv + kvh]);
+        const float v_sc = a.v_scale[(long)chunk * a.Hkv + kvh];
+        if constexpr (!POW2) c = c_q * k_sc;                             // per-lane score scale inside this piece
+        shift = uni(P_SHIFT + __builtin_amdgcn_logf(v_sc) - log2_vmax);  // <= 8
+        unshift = uni(__builtin_amdgcn_exp2f(-shift));
+        e_k = (__builtin_bit_cast(int, k_sc) >> 23) & 0xff;  // E8M0 code of a power-of-two key scale
+      }
 
       auto read_k = [&](int t, int kk) -> i32x8 {
         const int o = (base_k ^ (kk << 6)) + t * 4096;
@@ -268,7 +295,6 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       ka[0] = read_k(0, 0);
       ka[1] = read_k(0, 1);
       if constexpr (POW2) {
-        const int e_k = (__builtin_bit_cast(int, k_sc) >> 23) & 0xff;
         if (shift != cur_shift) {  // a new scale chunk (wave-uniform): re-base the accumulator offset
           const float ds = shift - cur_shift;
 #pragma unroll
@@ -383,7 +409,14 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
     }
     k0 = k1;
     pe = pe1;
-    buf ^= 1;
+    chunk = chunk1;
+    new_piece = new_piece1;
+  };
+  while (true) {  // unrolled by two: every LDS buffer index is a compile-time constant
+    tile_step(std::integral_constant<int, 0>{});
+    if (k0 >= ke) break;
+    tile_step(std::integral_constant<int, 1>{});
+    if (k0 >= ke) break;
   }
 
   if (!wave_on) return;

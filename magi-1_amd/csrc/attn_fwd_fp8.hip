@@ -342,7 +342,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         const bool raise = first || over > 0.f;
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
           const float delta = raise ? over : 0.f;
-          const float alpha = __builtin_amdgcn_exp2f(-delta);
+          const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);  // nothing to rescale on the first tile
           m_run += delta;
           l_run *= alpha;
 #pragma unroll
@@ -366,7 +366,9 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2]);
           const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3]);
           psum += (p0 + p1) + (p2 + p3);
-          int u = 0;
+          // v_cvt_pk_fp8_f32 keeps the other half of its destination: start from p0's register (its high half is
+          // overwritten by the second conversion) instead of a zeroed one
+          int u = __builtin_bit_cast(int, p0);
           u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
           u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
           pb[n] = u;
@@ -384,7 +386,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2] * c - mc);
           const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3] * c - mc);
           psum += (p0 + p1) + (p2 + p3);
-          int u = 0;
+          int u = __builtin_bit_cast(int, p0);  // see the power-of-two branch
           u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
           u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
           pb[n] = u;

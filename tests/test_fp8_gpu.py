@@ -101,6 +101,38 @@ def test_fp8_pow2_prescaled_mode(dev, L, dn, sp, Hq, Hkv, C):
     assert (lse.cpu() - lse_ref).abs().max() < 1e-3
 
 
+@pytest.mark.parametrize("pow2", [False, True])
+def test_fp8_scores_far_below_zero_from_the_first_tile(dev, pow2):
+    """All scores near -260 in base-2 units (q and k anti-parallel): the running maximum starts far below its
+    initial value, and the first tile's rescale factor 2^(+260) must not reach the (empty) accumulators."""
+    import math
+
+    g = torch.Generator().manual_seed(77)
+    T, Hq, Hkv, D = 200, 2, 1, 128
+    sign = torch.where(torch.rand(D, generator=g) < 0.5, -1.0, 1.0)
+    q = (4.0 * sign + 0.05 * torch.randn(T, Hq, D, generator=g)).bfloat16()
+    k = (-4.0 * sign + 0.05 * torch.randn(T, Hkv, D, generator=g)).bfloat16()
+    v = torch.randn(T, Hkv, D, generator=g).bfloat16()
+    qr, kr = [[0, T]], [[0, T]]
+    cs = D ** -0.5 * math.log2(math.e)
+    assert (q[0, 0].float() @ k[0, 0].float()).item() * cs < -200
+    q8, qs = M.quantize_fp8(q.to(dev), T, premul=cs if pow2 else 1.0, pow2_scales=pow2)
+    k8, ks = M.quantize_fp8(k.to(dev), T, pow2_scales=pow2)
+    v8, vs = M.quantize_fp8(v.to(dev), T, pow2_scales=pow2)
+    tq = torch.tensor(qr, dtype=torch.int32, device=dev)
+    tk = torch.tensor(kr, dtype=torch.int32, device=dev)
+    out, lse = M.range_attention(q8, k8, v8, tq, tk, T, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=T,
+                                 fp8_pow2_prescaled=pow2)
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    qd = O.dequantize_per_head_chunk(q8.cpu(), qs.cpu(), T)
+    kd = O.dequantize_per_head_chunk(k8.cpu(), ks.cpu(), T)
+    vd = O.dequantize_per_head_chunk(v8.cpu(), vs.cpu(), T)
+    ref = O.range_attention(qd / cs * D ** -0.5, kd, vd, qr, kr, softmax_scale=1.0) if pow2 else O.range_attention(qd, kd, vd, qr, kr)
+    err, cos = _per_head(out, ref)
+    # near-uniform attention: the rows are means of 200 V rows (|o| ~ 0.07), so the cosine bound is the looser one
+    assert err <= 4e-2 and cos >= 0.998, (err, cos)
+
+
 def test_fp8_uneven_scales_and_two_segments(dev):
     """Chunks with very different magnitudes (the per-chunk scales must be honoured, including the
     relative V scale folded into the exponent) and a key axis split over two buffers."""

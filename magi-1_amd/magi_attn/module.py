@@ -19,7 +19,8 @@ What differs is what happens underneath:
     [cache prefix | side buffer] as one key axis.
 
 The linear projections and the input LayerNorm are plain library GEMMs / ops (torch on
-rocBLAS / hipBLASLt); they are not part of this library.
+rocBLAS / hipBLASLt); they are not part of this library.  forward() runs the four projections
+q, k, v, qx as ONE GEMM over a shared weight buffer (CustomLayerNormLinear.forward_qkvx).
 """
 from __future__ import annotations
 
@@ -71,7 +72,14 @@ class FusedLayerNorm(torch.nn.Module):
 
 
 class CustomLayerNormLinear(torch.nn.Module):
-    """Input LayerNorm + the four projections q, qx, k, v (dit_module.py:390-425)."""
+    """Input LayerNorm + the four projections q, qx, k, v (dit_module.py:390-425).
+
+    The four weights keep the reference's parameter names (q.weight, qx.weight, k.weight, v.weight) but live
+    side by side in ONE buffer, rows ordered [q | k | v | qx], so forward_qkvx() is a single GEMM over the
+    normalised input instead of four (the input, 1 GB at the 720p shape, is read once, and the fused prologue
+    takes q / k / v as row-strided views of the one result).  Loading a state dict copies into the shared buffer
+    in place; after anything that re-allocates the parameters (.to(), .bfloat16()) the buffer is rebuilt on the
+    next call."""
 
     def __init__(self, input_size: int, output_size_q: int, output_size_kv: int, eps: float = 1e-6,
                  dtype=torch.bfloat16, device=None):
@@ -81,6 +89,42 @@ class CustomLayerNormLinear(torch.nn.Module):
         self.qx = torch.nn.Linear(input_size, output_size_q, bias=False, dtype=dtype, device=device)
         self.k = torch.nn.Linear(input_size, output_size_kv, bias=False, dtype=dtype, device=device)
         self.v = torch.nn.Linear(input_size, output_size_kv, bias=False, dtype=dtype, device=device)
+        self._fuse_weights()
+
+    def _projections(self):
+        return (self.q, self.k, self.v, self.qx)  # row order of the shared buffer
+
+    def _fuse_weights(self) -> torch.Tensor:
+        """Move the four weights into one [2*out_q + 2*out_kv, in] buffer and make each parameter a view of it."""
+        ws = [m.weight.data for m in self._projections()]
+        fused = torch.cat(ws, dim=0)
+        row = 0
+        for m, w in zip(self._projections(), ws):
+            m.weight.data = fused[row:row + w.shape[0]]
+            row += w.shape[0]
+        return fused
+
+    def fused_weight(self) -> torch.Tensor:
+        """The [q | k | v | qx] weight as one tensor (rebuilt first if the parameters no longer share a buffer)."""
+        ws = [m.weight.data for m in self._projections()]
+        base = ws[0]
+        ptr = base.data_ptr()
+        shared = True
+        for w in ws:
+            shared &= (w.data_ptr() == ptr and w.is_contiguous() and w.dtype == base.dtype and w.device == base.device
+                       and w.untyped_storage().data_ptr() == base.untyped_storage().data_ptr())
+            ptr += w.numel() * w.element_size()
+        if not shared:
+            return self._fuse_weights()
+        rows = sum(w.shape[0] for w in ws)
+        return base.as_strided((rows, base.shape[1]), (base.shape[1], 1))
+
+    def forward_qkvx(self, hidden_states):
+        """One GEMM for all four projections of the (already normalised) input -> views (q, k, v, qx) of one
+        [..., 2*out_q + 2*out_kv] result."""
+        y = torch.nn.functional.linear(hidden_states, self.fused_weight())
+        oq, okv = self.q.weight.shape[0], self.k.weight.shape[0]
+        return y[..., :oq], y[..., oq:oq + okv], y[..., oq + okv:oq + 2 * okv], y[..., oq + 2 * okv:]
 
     def forward_ln(self, hidden_states):
         return self.layer_norm(hidden_states)
@@ -181,16 +225,21 @@ class FullyParallelAttention(torch.nn.Module):
         D = self.hidden_size_per_attention_head
         return q, kv[..., :D].contiguous(), kv[..., D:].contiguous()
 
-    def _fused_qkv(self, mixed_qqkv, cos_emb, sin_emb, want_q=True, kv_out=None, n_cache_rows=None, kv_tail=None):
+    def _fused_qkv(self, mixed_qqkv, cos_emb, sin_emb, want_q=True, kv_out=None, n_cache_rows=None, kv_tail=None,
+                   raw=None):
+        """raw: (q_raw, k_raw, v_raw) already projected (views of forward_qkvx's result), else projected here."""
         sq, b = mixed_qqkv.shape[0], mixed_qqkv.shape[1]
         S = sq * b
         Hq, Hkv = self.num_attention_heads, self.num_query_groups_per_partition
-        k_raw = self.linear_qkv.forward_k(mixed_qqkv).reshape(S, -1)
-        v_raw = self.linear_qkv.forward_v(mixed_qqkv).reshape(S, -1)
-        if want_q:
-            q_raw = self.linear_qkv.forward_q(mixed_qqkv).reshape(S, -1)
+        if raw is not None:
+            q_raw, k_raw, v_raw = (t.reshape(S, -1) for t in raw)  # [sq, b, n] row-strided: still a view
         else:
-            q_raw = k_raw[:, :0]
+            k_raw = self.linear_qkv.forward_k(mixed_qqkv).reshape(S, -1)
+            v_raw = self.linear_qkv.forward_v(mixed_qqkv).reshape(S, -1)
+            if want_q:
+                q_raw = self.linear_qkv.forward_q(mixed_qqkv).reshape(S, -1)
+            else:
+                q_raw = k_raw[:, :0]
         rope = torch.cat([sin_emb, cos_emb], dim=-1).float().contiguous()
         gq, bq = self.q_layernorm.gamma_beta_fp32()
         gk, bk = self.k_layernorm.gamma_beta_fp32()
@@ -198,10 +247,11 @@ class FullyParallelAttention(torch.nn.Module):
                                   eps=self.eps, kv_out=kv_out, n_cache_rows=n_cache_rows, kv_tail=kv_tail, batch=b)
         return (q if want_q else None), (kv if tail is None else (kv, tail))
 
-    def get_xqkv(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor):
-        """Cross-attention q (normed) and k (normed) / v from the text states; dit_module.py:1005-1021."""
+    def get_xqkv(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor, qx_raw: Optional[torch.Tensor] = None):
+        """Cross-attention q (normed) and k (normed) / v from the text states; dit_module.py:1005-1021.
+        qx_raw: the qx projection when the caller already has it (forward_qkvx), else projected here."""
         D = self.hidden_size_per_attention_head
-        qx = self.linear_qkv.forward_qx(mixed_qqkv)  # [sq, b, Hq*D]
+        qx = self.linear_qkv.forward_qx(mixed_qqkv) if qx_raw is None else qx_raw  # [sq, b, Hq*D]
         qx = qx.transpose(0, 1).reshape(qx.shape[0] * qx.shape[1], -1, D)  # "(b sq) hn hd"
         gq, bq = self.q_layernorm_xattn.gamma_beta_fp32()
         qx = head_norm(qx, gq, bq, self.eps)
@@ -292,6 +342,10 @@ class FullyParallelAttention(torch.nn.Module):
         sq = hidden_states.shape[0]
         D = self.hidden_size_per_attention_head
         mixed_qqkv = self.linear_qkv.forward_ln(hidden_states)
+        # all four projections in one GEMM; q / k / v feed the fused prologue as row-strided views of its result
+        q_raw, k_raw, v_raw, qx_raw = self.linear_qkv.forward_qkvx(mixed_qqkv)
+        raw = (q_raw, k_raw, v_raw)
+        get_xqkv = lambda m, y: self.get_xqkv(m, y, qx_raw=qx_raw)
         p = meta_args.core_attn_params
         Hq = self.num_attention_heads
         fused = None
@@ -304,7 +358,7 @@ class FullyParallelAttention(torch.nn.Module):
         use_cache = inference_params is not None and (
             meta_args.extract_prefix_video_feature or meta_args.fwd_extra_1st_chunk or meta_args.slice_point > 0)
         if not use_cache:
-            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb)
+            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw)
             core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst)
         else:
             if bs != 1 or inference_params.max_batch_size != 1:
@@ -322,7 +376,7 @@ class FullyParallelAttention(torch.nn.Module):
             if n_keep < S:
                 tail = torch.empty(S - n_keep, cache.shape[1], cache.shape[2], dtype=cache.dtype, device=cache.device)
             q, _ = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, kv_out=cache[start:], n_cache_rows=n_keep,
-                                   kv_tail=tail)
+                                   kv_tail=tail, raw=raw)
             split = start + n_keep
             kc, vc = cache[:split, :, :D], cache[:split, :, D:]
             if tail is None:
@@ -333,10 +387,10 @@ class FullyParallelAttention(torch.nn.Module):
                                           k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, out=core_dst,
                                           return_lse=False)
         if fused is not None:
-            self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, self.get_xqkv, out=cross_dst)
+            self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, get_xqkv, out=cross_dst)
             return fused
         core_attn_out = core.view(sq, bs, -1)
-        xattn_out = self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, self.get_xqkv)
+        xattn_out = self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, get_xqkv)
         if proj_layout:
             return attn_linear_proj_input(core_attn_out, xattn_out)
         return core_attn_out, xattn_out

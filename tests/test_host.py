@@ -180,3 +180,30 @@ def test_kv_cache_arena_views_accounting_and_errors():
         KVCacheArena(48, 259200, 8, device="cpu", memory_budget_bytes=1 << 30)
     with pytest.raises(ValueError):
         KVCacheArena(1, 8, 1, device="cpu", kv_offload=True)
+
+
+def test_projection_weights_share_one_buffer():
+    """q / k / v / qx keep the reference's parameter names but are rows of one buffer, so one GEMM serves all four;
+    the sharing survives load_state_dict and is re-established after a dtype / device move."""
+    from magi_attn.module import CustomLayerNormLinear
+
+    torch.manual_seed(0)
+    m = CustomLayerNormLinear(64, 48, 16, dtype=torch.float32)
+    assert sorted(n for n, _ in m.named_parameters()) == ["k.weight", "layer_norm.bias", "layer_norm.weight", "q.weight",
+                                                          "qx.weight", "v.weight"]
+    w = m.fused_weight()
+    assert w.shape == (128, 64) and w.data_ptr() == m.q.weight.data_ptr()
+    x = torch.randn(5, 1, 64)
+    q, k, v, qx = m.forward_qkvx(x)
+    for got, lin in ((q, m.forward_q), (k, m.forward_k), (v, m.forward_v), (qx, m.forward_qx)):
+        assert torch.allclose(got, lin(x), atol=1e-6)
+    sd = {n: torch.randn_like(t) for n, t in m.state_dict().items()}
+    m.load_state_dict(sd)
+    w2 = m.fused_weight()
+    assert w2.data_ptr() == w.data_ptr()  # copied in place, still shared
+    assert torch.equal(w2, torch.cat([sd["q.weight"], sd["k.weight"], sd["v.weight"], sd["qx.weight"]]))
+    m = m.to(torch.bfloat16)  # re-allocates every parameter: the buffer is rebuilt on the next call
+    w3 = m.fused_weight()
+    assert w3.dtype == torch.bfloat16 and w3.data_ptr() == m.q.weight.data_ptr()
+    assert m.k.weight.data_ptr() == w3.data_ptr() + 48 * 64 * 2
+    assert torch.equal(w3[80:], sd["qx.weight"].bfloat16())

@@ -128,7 +128,7 @@ int magi_attn_fwd(const magi_attn_args* args, void* stream);
  * rope  [S / batch, 2*R2] fp32, sin in the first R2 columns, cos in the last R2 (dit_module.py:770, 1147);
  *       rotary_dim = 2*R2 <= D; NULL disables rotary
  * gq,bq,gk,bk  fp32 [D] norm parameters (gamma stored zero-centred); b* may be NULL
- * q_out [S, Hq, D] bf16 contiguous (or fp8 with q_scale_out, see below)
+ * q_out [S, Hq, D] bf16 contiguous
  * kv_out  row 0 of the destination for the first n_cache_rows tokens: [*, Hkv, 2D] with token
  *         stride kv_stride_t; K goes to [..., 0:D], V to [..., D:2D]
  * kv_tail destination of tokens >= n_cache_rows (same layout, row index t - n_cache_rows); may be

@@ -58,3 +58,29 @@ class KVCacheArena:
         for i, n in enumerate(numbers):
             inference_params.key_value_memory_dict[n] = self.buffer[i]
         return inference_params.key_value_memory_dict
+
+
+class Fp8KVCache:
+    """One layer's KV cache for the fp8 attention path: K and V as e4m3 bytes [max_sequence_length, Hkv, D] each,
+    plus one power-of-two fp32 scale per (chunk of `chunk_tokens` tokens, KV head).  A chunk of the cache is a
+    video chunk (`clip_token_nums` tokens, the unit in which the pipeline appends and re-reads KV,
+    inference/model/dit/dit_module.py:905-929), so appending a chunk never re-scales rows already stored.
+    Half the bytes of the bf16 cache: 0.53 GB per layer at the 24B / 720p shape.
+
+    The reference has no fp8 attention; this object takes the place of the tensor it keeps in
+    `InferenceParams.key_value_memory_dict[layer_number]` when the layer runs with attention_dtype="fp8"."""
+
+    def __init__(self, max_sequence_length: int, num_query_groups: int, chunk_tokens: int, head_dim: int = 128,
+                 device=None):
+        if min(max_sequence_length, num_query_groups, chunk_tokens) <= 0:
+            raise ValueError("all sizes must be positive")
+        self.chunk_tokens = chunk_tokens
+        n_chunks = (max_sequence_length + chunk_tokens - 1) // chunk_tokens
+        self.k = torch.zeros(max_sequence_length, num_query_groups, head_dim, dtype=torch.float8_e4m3fn, device=device)
+        self.v = torch.zeros_like(self.k)
+        self.k_scale = torch.ones(n_chunks, num_query_groups, dtype=torch.float32, device=device)
+        self.v_scale = torch.ones_like(self.k_scale)
+
+    @property
+    def max_sequence_length(self) -> int:
+        return self.k.shape[0]

@@ -261,10 +261,14 @@ def head_norm(x: torch.Tensor, gamma, beta, eps: float = 1e-6, norm_kind: int = 
     return y
 
 
-def quantize_fp8(x: torch.Tensor, chunk_tokens: int, premul: float = 1.0, pow2_scales: bool = False):
+def quantize_fp8(x: torch.Tensor, chunk_tokens: int, premul: float = 1.0, pow2_scales: bool = False,
+                 out: Optional[torch.Tensor] = None, scales_out: Optional[torch.Tensor] = None):
     """x [T, H, 128] bf16 (strided heads allowed) -> (y [T, H, 128] float8_e4m3fn, scales [ceil(T/chunk), H] fp32)
     with x * premul ~= y * scales[t // chunk_tokens, h]: per-(chunk, head) absmax * |premul| / 448 (rounded up to a
     power of two with pow2_scales), saturating OCP e4m3fn.
+
+    out / scales_out: contiguous destinations (e.g. the rows of an fp8 KV cache at the write position and the
+    matching rows of its scale table) instead of fresh tensors.
 
     For the fast attention mode quantise q with premul = softmax_scale * log2(e) and q, k, v with pow2_scales,
     then pass fp8_pow2_prescaled=True to range_attention."""
@@ -273,8 +277,13 @@ def quantize_fp8(x: torch.Tensor, chunk_tokens: int, premul: float = 1.0, pow2_s
         raise TypeError("x must be bf16")
     T, H, D = x.shape
     n_chunks = (T + chunk_tokens - 1) // chunk_tokens
-    y = torch.empty((T, H, D), dtype=torch.float8_e4m3fn, device=x.device)
-    scales = torch.empty((n_chunks, H), dtype=torch.float32, device=x.device)
+    y = torch.empty((T, H, D), dtype=torch.float8_e4m3fn, device=x.device) if out is None else out
+    scales = torch.empty((n_chunks, H), dtype=torch.float32, device=x.device) if scales_out is None else scales_out
+    if y.dtype != torch.float8_e4m3fn or tuple(y.shape) != (T, H, D) or not y.is_contiguous() or y.device != x.device:
+        raise ValueError("out must be a contiguous float8_e4m3fn [T, H, 128] tensor on x's device")
+    if (scales.dtype != torch.float32 or tuple(scales.shape) != (n_chunks, H) or not scales.is_contiguous()
+            or scales.device != x.device):
+        raise ValueError("scales_out must be a contiguous fp32 [ceil(T / chunk_tokens), H] tensor on x's device")
     with torch.cuda.device(x.device):
         L.check(L.lib().magi_quantize_fp8(x.data_ptr(), x.stride(0), x.stride(1), y.data_ptr(), scales.data_ptr(), T, H, D,
                                           int(chunk_tokens), float(premul), int(pow2_scales), _stream()))

@@ -28,8 +28,11 @@ from typing import Callable, Optional, Tuple
 
 import torch
 
+import math
+
 from . import _lib as L
-from .functional import head_norm, qk_prologue, range_attention
+from .cache import Fp8KVCache
+from .functional import head_norm, qk_prologue, quantize_fp8, range_attention
 from .params import InferenceParams, ModelMetaArgs, PackedCrossAttnParams
 
 
@@ -145,10 +148,17 @@ class CustomLayerNormLinear(torch.nn.Module):
 class FullyParallelAttention(torch.nn.Module):
     def __init__(self, hidden_size: int, num_attention_heads: int, num_query_groups: int, kv_channels: int = 128,
                  layer_number: int = 0, layernorm_epsilon: float = 1e-6, apply_layernorm_1p: bool = True,
-                 xattn_cond_hidden_ratio: float = 1.0, params_dtype=torch.bfloat16, device=None):
+                 xattn_cond_hidden_ratio: float = 1.0, params_dtype=torch.bfloat16, device=None,
+                 attention_dtype: str = "bf16"):
+        """attention_dtype "fp8" (not in the reference, which has no fp8 attention) runs the self-attention on
+        e4m3 operands with per-(video chunk, head) power-of-two scales and keeps the KV cache in that form
+        (Fp8KVCache); the cross attention and everything else stay in bf16."""
         super().__init__()
         if kv_channels != 128:
             raise NotImplementedError("head_dim 128 only")
+        if attention_dtype not in ("bf16", "fp8"):
+            raise ValueError("attention_dtype must be 'bf16' or 'fp8'")
+        self.attention_dtype = attention_dtype
         self.layer_number = layer_number
         self.hidden_size_per_attention_head = kv_channels
         self.num_attention_heads = num_attention_heads
@@ -181,6 +191,66 @@ class FullyParallelAttention(torch.nn.Module):
             d[self.layer_number] = self._allocate_key_and_value_memory(
                 inference_params.max_sequence_length, inference_params.max_batch_size, dtype)
         return d[self.layer_number]
+
+    def _cache_fp8(self, inference_params: InferenceParams, chunk_tokens: int) -> Fp8KVCache:
+        d = inference_params.key_value_memory_dict
+        if self.layer_number not in d:
+            d[self.layer_number] = Fp8KVCache(inference_params.max_sequence_length * inference_params.max_batch_size,
+                                              self.num_query_groups_per_partition, chunk_tokens,
+                                              self.hidden_size_per_attention_head,
+                                              device=self.linear_qkv.q.weight.device)
+        cache = d[self.layer_number]
+        if not isinstance(cache, Fp8KVCache) or cache.chunk_tokens != chunk_tokens:
+            raise ValueError("this layer's cache entry is not an Fp8KVCache with chunk_tokens == clip_token_nums")
+        return cache
+
+    def _core_attention_fp8(self, q: torch.Tensor, kv_new: torch.Tensor, inference_params: Optional[InferenceParams],
+                            meta_args: ModelMetaArgs, use_cache: bool, out: Optional[torch.Tensor]) -> torch.Tensor:
+        """Self-attention on e4m3 operands: q [S, Hq, D] and kv_new [S, Hkv, 2D] are the prologue's bf16 results.
+        Scale chunks are video chunks (clip_token_nums tokens), so the cache rules of the bf16 path
+        (dit_module.py:905-931: append at slice_point, keep nothing when update_kv_cache is False, keep all but
+        the last chunk under distill_nearly_clean_chunk) carry over chunk by chunk."""
+        D = self.hidden_size_per_attention_head
+        Lc = meta_args.clip_token_nums
+        p = meta_args.core_attn_params
+        S = q.shape[0]
+        q8, qs = quantize_fp8(q, Lc, premul=D ** -0.5 * math.log2(math.e), pow2_scales=True)
+        k_new, v_new = kv_new[..., :D], kv_new[..., D:]
+        kw = dict(q_scale=qs, scale_chunk_tokens=Lc, fp8_pow2_prescaled=True, out=out, return_lse=False)
+        if not use_cache:
+            k8, ks = quantize_fp8(k_new, Lc, pow2_scales=True)
+            v8, vs = quantize_fp8(v_new, Lc, pow2_scales=True)
+            o, _ = range_attention(q8, k8, v8, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k, k_scale=ks, v_scale=vs,
+                                   **kw)
+            return o
+        cache = self._cache_fp8(inference_params, Lc)
+        start = meta_args.slice_point * Lc
+        if inference_params.update_kv_cache:
+            n_keep = S - Lc if meta_args.distill_nearly_clean_chunk else S
+        else:
+            n_keep = 0
+        if S % Lc or n_keep < 0:
+            raise ValueError("the fp8 path works on whole video chunks")
+        if start + n_keep > cache.max_sequence_length:
+            raise ValueError("KV cache overflow")
+        c0 = start // Lc
+        if n_keep:
+            rows, chunks = slice(start, start + n_keep), slice(c0, c0 + n_keep // Lc)
+            quantize_fp8(k_new[:n_keep], Lc, pow2_scales=True, out=cache.k[rows], scales_out=cache.k_scale[chunks])
+            quantize_fp8(v_new[:n_keep], Lc, pow2_scales=True, out=cache.v[rows], scales_out=cache.v_scale[chunks])
+        split = start + n_keep
+        if n_keep == S:
+            o, _ = range_attention(q8, cache.k[:split], cache.v[:split], p.q_range, p.k_range, p.max_seqlen_q,
+                                   p.max_seqlen_k, k_scale=cache.k_scale, v_scale=cache.v_scale, **kw)
+            return o
+        # rows that must not be persisted: a side buffer behind the cached prefix, its scales behind the prefix's
+        k2, k2s = quantize_fp8(k_new[n_keep:], Lc, pow2_scales=True)
+        v2, v2s = quantize_fp8(v_new[n_keep:], Lc, pow2_scales=True)
+        ks = torch.cat([cache.k_scale[:split // Lc], k2s])
+        vs = torch.cat([cache.v_scale[:split // Lc], v2s])
+        o, _ = range_attention(q8, cache.k[:split], cache.v[:split], p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
+                               k2=k2, v2=v2, k_split=split, k_scale=ks, v_scale=vs, **kw)
+        return o
 
     # --------------------------------------------------- reference-shaped pieces
     def _prologue_single(self, raw: torch.Tensor, which: str, cos_emb, sin_emb) -> torch.Tensor:
@@ -357,7 +427,12 @@ class FullyParallelAttention(torch.nn.Module):
 
         use_cache = inference_params is not None and (
             meta_args.extract_prefix_video_feature or meta_args.fwd_extra_1st_chunk or meta_args.slice_point > 0)
-        if not use_cache:
+        if self.attention_dtype == "fp8":
+            if bs != 1 or (use_cache and inference_params.max_batch_size != 1):
+                raise ValueError("the fp8 self-attention runs at batch 1")
+            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw)
+            core = self._core_attention_fp8(q, kv, inference_params, meta_args, use_cache, core_dst)
+        elif not use_cache:
             q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw)
             core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst)
         else:

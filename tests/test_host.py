@@ -207,3 +207,18 @@ def test_projection_weights_share_one_buffer():
     assert w3.dtype == torch.bfloat16 and w3.data_ptr() == m.q.weight.data_ptr()
     assert m.k.weight.data_ptr() == w3.data_ptr() + 48 * 64 * 2
     assert torch.equal(w3[80:], sd["qx.weight"].bfloat16())
+
+
+def test_fp8_kv_cache_shapes_and_layer_option():
+    from magi_attn.cache import Fp8KVCache
+    from magi_attn.module import FullyParallelAttention
+
+    c = Fp8KVCache(10 * 24, 2, 24)
+    assert c.k.shape == c.v.shape == (240, 2, 128) and c.k.dtype == torch.float8_e4m3fn
+    assert c.k_scale.shape == c.v_scale.shape == (10, 2) and c.max_sequence_length == 240
+    assert Fp8KVCache(25, 1, 24).k_scale.shape == (2, 1)  # a partial last chunk has a scale row too
+    with pytest.raises(ValueError):
+        Fp8KVCache(0, 2, 24)
+    with pytest.raises(ValueError):
+        FullyParallelAttention(64, 2, 1, attention_dtype="fp4")
+    assert FullyParallelAttention(64, 2, 1, attention_dtype="fp8").attention_dtype == "fp8"

@@ -323,3 +323,69 @@ def test_layer_with_arena_backed_cache(dev):
         assert torch.equal(c0, c1) and torch.equal(x0, x1)
     assert torch.equal(outs[0][1][: 4 * L], outs[1][1][: 4 * L])
     assert torch.isnan(arena.layer(2)).all() and torch.isnan(arena.layer(4)).all()  # other layers untouched
+
+
+def test_layer_with_fp8_self_attention_and_fp8_cache(dev):
+    """attention_dtype="fp8": same schedule as above through two layers with identical weights, one bf16 and one
+    fp8.  The reference has no fp8 attention (parity unpinned by it); the bf16 layer, itself checked against the
+    oracle above, is the yardstick: per step cosine >= 0.998 and max-abs <= 2^-5 max|V| on the self-attention
+    output, bit-identical cross-attention output, and a cache that dequantises to the bf16 cache within e4m3
+    rounding (2^-4 relative, per-(chunk, head) scale)."""
+    from magi_attn.cache import Fp8KVCache
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+
+    hidden, Hq, Hkv, D = 256, 6, 2, 128
+    fr, H, W = 2, 3, 4
+    L = fr * H * W
+    n_chunks = 6
+    ref_layer = _make_layer(dev, hidden, Hq, Hkv, seed=5)
+    torch.manual_seed(5)
+    fp8_layer = MOD.FullyParallelAttention(hidden, Hq, Hkv, layer_number=3, device=dev, attention_dtype="fp8")
+    fp8_layer.load_state_dict(ref_layer.state_dict())
+    rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
+    ip_ref, ip_fp8 = P.InferenceParams(1, n_chunks * L), P.InferenceParams(1, n_chunks * L)
+    g = torch.Generator().manual_seed(6)
+    #        sp dn update distill extra has_ip
+    steps = [(0, 2, True, False, True, True),
+             (0, 3, True, True, True, True),
+             (2, 3, False, False, False, True),
+             (2, 3, True, False, False, True),
+             (1, 4, True, True, True, True),
+             (3, 3, False, False, True, True),
+             (0, 2, False, False, False, False)]
+    for sp, dn, update, distill, extra, has_ip in steps:
+        S = dn * L
+        hs = torch.randn(S, 1, hidden, generator=g).bfloat16().to(dev)
+        lens = torch.randint(0, 9, (dn,), generator=g)
+        mask = (torch.arange(8)[None] < lens[:, None]).float().view(dn, 1, 1, 8)
+        y = (torch.randn(int(lens.sum()), hidden, generator=g) * 0.5).bfloat16().to(dev)
+        k_range = R.generate_default_kvrange(sp, dn, L) if has_ip else R.generate_kv_range_for_uncondition(dn, L)
+        q_range = R.q_ranges_from_chunks(dn, L)
+        meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=sp, denoising_range_num=dn,
+                               range_num=sp + dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=extra,
+                               distill_nearly_clean_chunk=distill, clip_token_nums=L, enable_cuda_graph=False,
+                               core_attn_params=P.build_core_attn_params(q_range.to(dev), k_range.to(dev), L),
+                               cross_attn_params=P.build_cross_attn_params(mask.to(dev), L, 8))
+        rope = rope_mod.get_embed_for_forward(dn * fr, H, W, sp, dn)
+        ip_ref.update_kv_cache = ip_fp8.update_kv_cache = update
+        with torch.no_grad():
+            core_ref, xo_ref = ref_layer(hs, y, ip_ref if has_ip else None, rope, meta)
+            core, xo = fp8_layer(hs, y, ip_fp8 if has_ip else None, rope, meta)
+            vmax = ref_layer.linear_qkv.forward_v(ref_layer.linear_qkv.forward_ln(hs)).float().abs().max().item()
+        assert torch.equal(xo, xo_ref)
+        a, b = core.double().flatten(), core_ref.double().flatten()
+        cos = (a @ b / (a.norm() * b.norm())).item()
+        err = (a - b).abs().max().item()
+        if has_ip and ip_ref.key_value_memory_dict:
+            vmax = max(vmax, ip_ref.key_value_memory_dict[3][..., D:].float().abs().max().item())
+        assert cos >= 0.998 and err <= 2 ** -5 * vmax, ((sp, dn, update, distill, extra), cos, err, vmax)
+        if has_ip and (extra or sp > 0) and update:
+            keep = S - L if distill else S
+            cache = ip_fp8.key_value_memory_dict[3]
+            assert isinstance(cache, Fp8KVCache)
+            rows = slice(sp * L, sp * L + keep)
+            sc = lambda t: t[sp:sp + keep // L].repeat_interleave(L, dim=0)[:, :, None]
+            want = ip_ref.key_value_memory_dict[3][rows].float()
+            for got, ref_half in ((cache.k[rows].float() * sc(cache.k_scale), want[..., :D]),
+                                  (cache.v[rows].float() * sc(cache.v_scale), want[..., D:])):
+                assert ((got - ref_half).abs() <= ref_half.abs() * 2 ** -4 + 2 ** -9 * ref_half.abs().max()).all()

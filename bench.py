@@ -38,7 +38,7 @@ WORKLOADS = {
 }
 
 
-def build_inputs(name, dev, seed=1234):
+def build_inputs(name, dev, seed=1234, kv_window="default"):
     import magi_attn as M
     from magi_attn.rope import LearnableRotaryEmbeddingCat
 
@@ -69,7 +69,12 @@ def build_inputs(name, dev, seed=1234):
     from magi_attn import ranges as R
 
     inp["q_ranges"] = R.q_ranges_from_chunks(dn, L, device=dev)
-    inp["k_ranges"] = R.generate_default_kvrange(sp, dn, L, device=dev)
+    if kv_window == "default":  # every chunk attends to all chunks up to itself (the configuration the metric is quoted on)
+        kr = R.generate_default_kvrange(sp, dn, L)
+    else:  # the shipped sliding window: noise2clean_kvrange [5, 4, 3, 2] over 32 steps, chunks 8 steps apart
+        kr = R.generate_noise2clean_kvrange(sp, dn, L, [5, 4, 3, 2], 1, [8 * (dn - 1 - j) for j in range(dn)][:dn], 32)
+    inp["k_ranges_host"] = kr.numpy()
+    inp["k_ranges"] = kr.to(dev)
     # T5 side: valid lengths uniform in [20, 800] per chunk, K | V interleaved per head as the projection emits them
     rs = np.random.default_rng(seed)
     lens = rs.integers(20, 801, size=dn)
@@ -82,7 +87,7 @@ def build_inputs(name, dev, seed=1234):
 
 def flops_of(inp):
     L, dn, sp, Hq, D = inp["L"], inp["dn"], inp["sp"], inp["Hq"], inp["D"]
-    core = 4.0 * D * Hq * sum(L * (sp + j + 1) * L for j in range(dn))
+    core = 4.0 * D * Hq * sum(L * float(e - b) for b, e in inp["k_ranges_host"])
     cross = 4.0 * D * Hq * float(sum(L * int(n) for n in inp["t5_lens"]))
     return core, cross
 
@@ -169,7 +174,7 @@ def cpu_baseline(inp, rows_per_chunk=6144):
     k = inp["cache"][:, :1, :D].float().cpu()
     v = inp["cache"][:, :1, D:].float().cpu()
     qr = np.array([[j * rows, (j + 1) * rows] for j in range(dn)])
-    kr = np.array([[0, (sp + j + 1) * L] for j in range(dn)])
+    kr = inp["k_ranges_host"]
     fl = O.attention_flops(qr, kr, G, D)
     torch.set_num_threads(os.cpu_count() if os.cpu_count() and os.cpu_count() <= 64 else torch.get_num_threads())
     t0 = time.perf_counter()
@@ -186,6 +191,8 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="720p-24B", choices=sorted(WORKLOADS))
+    ap.add_argument("--kv-window", default="default", choices=["default", "noise2clean"],
+                    help="key ranges: all chunks up to the query's own (default) or the shipped sliding window")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fp8", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -199,7 +206,7 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    inp = build_inputs(args.workload, dev)
+    inp = build_inputs(args.workload, dev, kv_window=args.kv_window)
     core_fl, cross_fl = flops_of(inp)
 
     for _ in range(args.warmup):
@@ -236,11 +243,12 @@ def main():
         "config": {"workload": f"{args.workload} layer-forward: prologue + chunk-causal attention "
                                f"(Q {inp['S']} tok x {inp['Hq']} heads over K/V {(inp['sp'] + inp['dn']) * inp['L']} tok x "
                                f"{inp['Hkv']} heads, d=128, {inp['sp']} cached + {inp['dn']} denoising chunks of {inp['L']}) "
-                               f"+ T5 cross-attention (lens {inp['t5_lens'].tolist()})",
+                               f"+ T5 cross-attention (lens {inp['t5_lens'].tolist()})"
+                               + ("" if args.kv_window == "default" else f", sliding-window key ranges {inp['k_ranges_host'].tolist()}"),
                    "core_flops": core_fl, "cross_flops": cross_fl},
         "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_kernel", "achieved": round(core_tflops, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(core_tflops / PEAK_BF16_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("core"), "ms": round(kern_ms["core"], 3)},
+                     "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("core") if args.kv_window == "default" else None, "ms": round(kern_ms["core"], 3)},
         "roofline_prologue": {"bound": "hbm", "kernel": "prologue_kernel", "achieved": round(pro_gbs, 1),
                               "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": round(pro_gbs / PEAK_HBM_GBS, 4),
                               "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get("prologue"),

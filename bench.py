@@ -35,6 +35,8 @@ WORKLOADS = {
     # name: (T_lat frames per chunk, H, W, denoise chunks, prefix chunks, Hq, Hkv)
     "720p-24B": (6, 45, 80, 4, 8, 48, 8),
     "480p-4.5B": (6, 30, 52, 4, 4, 24, 8),
+    # one rank's share of the 720p layer under an 8-way head split (one KV head with its 6 query heads, all tokens)
+    "720p-24B-head-share": (6, 45, 80, 4, 8, 6, 1),
 }
 
 

@@ -80,8 +80,6 @@ def range_attention(
     _check_thd(v, "v")
     Tq, Hq, D = q.shape
     Hkv = k.shape[1]
-    if k.stride() != v.stride() and (k.stride(0) != v.stride(0) or k.stride(1) != v.stride(1)):
-        pass  # independent strides are supported
     total_k = k.shape[0] if k2 is None else int(k_split) + k2.shape[0]
     if k2 is not None:
         _check_thd(k2, "k2")

@@ -321,3 +321,24 @@ def test_randomised_shapes_ranges_strides_and_splits(dev):
             _cmp(out[cov], ref[torch.tensor(covered)], f"case {case}")
         assert torch.count_nonzero(out[~cov]).item() == 0, f"case {case}: uncovered rows written"
         assert torch.isfinite(out).all()
+
+
+def test_repeated_launches_are_bit_identical(dev):
+    """The reference passes deterministic=torch.are_deterministic_algorithms_enabled() to its attention calls
+    (dit_module.py:1040, 1062, 1131).  This kernel has one writer per output row and no atomics, so every launch
+    gives the same bits, bf16 and fp8 alike, also when other work shares the GPU between the launches."""
+    L, dn, sp, Hq, Hkv = 700, 3, 2, 12, 4
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=99)
+    tq, tk = _ranges(dev, O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L))
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    first, lse0 = M.range_attention(qd, kd, vd, tq, tk, L)
+    q8, qs = M.quantize_fp8(qd, L)
+    k8, ks = M.quantize_fp8(kd, L)
+    v8, vs = M.quantize_fp8(vd, L)
+    first8, _ = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L)
+    for _ in range(3):
+        noise = torch.randn(1 << 20, device=dev).sum()  # unrelated work in between
+        again, lse = M.range_attention(qd, kd, vd, tq, tk, L)
+        again8, _ = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L)
+        assert torch.equal(again, first) and torch.equal(lse, lse0) and torch.equal(again8, first8)
+        del noise

@@ -20,7 +20,6 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 constexpr int D = 128;
 constexpr int THREADS = 256;
 constexpr int GROUPS = THREADS / 8;  // rows in flight per workgroup
-constexpr int TOK_PER_BLOCK = 1;
 
 __device__ __forceinline__ void unpack8(const u32x4 v, float* f) {
 #pragma unroll
@@ -72,6 +71,7 @@ __device__ __forceinline__ void norm16(float* x, const float* gam, const float* 
   }
 }
 
+template <int TPB>  // tokens that share a workgroup: 1, 2, 4 or 8
 __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArgs a) {
   __shared__ float s_par[4][D];  // gq, bq, gk, bk
   const int tid = threadIdx.x;
@@ -82,16 +82,21 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
   }
   __syncthreads();
 
-  const int j = tid & 7, grp = tid >> 3;
+  // The 32 row groups of the workgroup form tok_per_block teams of equal size, one token each, so that layers
+  // with few heads (e.g. one rank's share of a head-parallel split: 8 rows per token) still fill the workgroup.
+  const int j = tid & 7;
+  constexpr int gpt = GROUPS / TPB;  // row groups per token
+  const int team = TPB == 1 ? 0 : (tid >> 3) / gpt;  // (a constant keeps the token index in a scalar register)
+  const int grp = (tid >> 3) % gpt;
   const int nr = a.R2 >> 3;  // lanes that hold rotary pairs
   const bool rot_lane = j < nr;
   const int ea = rot_lane ? 8 * j : 2 * a.R2 + 16 * (j - nr);  // first element of vector A
   const int eb = rot_lane ? a.R2 + 8 * j : ea + 8;             // first element of vector B
   const int U = a.Hq + 2 * a.Hkv;
 
-  for (int tt = 0; tt < TOK_PER_BLOCK; ++tt) {
-    const int s = blockIdx.x * TOK_PER_BLOCK + tt;
-    if (s >= a.S) break;
+  {
+    const int s = blockIdx.x * TPB + team;
+    if (s >= a.S) return;
     float sn[8], cs[8];
     if (rot_lane && a.rope) {
       const float* rp = a.rope + (long)(s / a.batch) * (2 * a.R2);
@@ -107,7 +112,7 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
     }
     char* kvrow = (s < a.n_cache_rows) ? a.kv_out + (long)s * a.kv_stride_t
                                        : a.kv_tail + (long)(s - a.n_cache_rows) * a.kv_tail_stride_t;
-    for (int u = grp; u < U; u += GROUPS) {
+    for (int u = grp; u < U; u += gpt) {
       const char* src;
       char* dst;
       int kind;  // 0 = q, 1 = k, 2 = v
@@ -216,10 +221,19 @@ __global__ __launch_bounds__(THREADS) void rotary_kernel(const void* xin, const 
 
 }  // namespace
 
-hipError_t launch_prologue(const PrologueKernArgs& a, hipStream_t stream) {
-  if (a.S <= 0) return hipSuccess;
-  const unsigned grid = (unsigned)((a.S + TOK_PER_BLOCK - 1) / TOK_PER_BLOCK);
-  hipLaunchKernelGGL(prologue_kernel, dim3(grid), dim3(THREADS), 0, stream, a);
+hipError_t launch_prologue(const PrologueKernArgs& a_in, hipStream_t stream) {
+  if (a_in.S <= 0) return hipSuccess;
+  const PrologueKernArgs& a = a_in;
+  const int rows = a.Hq + 2 * a.Hkv;
+  int tpb = 1;
+  while (tpb < 8 && 2 * tpb * rows <= GROUPS) tpb *= 2;
+  const dim3 grid((unsigned)((a.S + tpb - 1) / tpb)), block(THREADS);
+  switch (tpb) {
+    case 1: hipLaunchKernelGGL(prologue_kernel<1>, grid, block, 0, stream, a); break;
+    case 2: hipLaunchKernelGGL(prologue_kernel<2>, grid, block, 0, stream, a); break;
+    case 4: hipLaunchKernelGGL(prologue_kernel<4>, grid, block, 0, stream, a); break;
+    default: hipLaunchKernelGGL(prologue_kernel<8>, grid, block, 0, stream, a); break;
+  }
   return hipGetLastError();
 }
 

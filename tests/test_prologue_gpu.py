@@ -39,7 +39,9 @@ def _inputs(S, Hq, Hkv, seed):
 
 
 @pytest.mark.parametrize("T,H,W,sp,dn,Hq,Hkv", [(2, 4, 6, 0, 1, 6, 2), (6, 5, 7, 2, 3, 24, 8), (4, 3, 3, 1, 2, 48, 8),
-                                                (2, 2, 2, 0, 2, 3, 1)])
+                                                (2, 2, 2, 0, 2, 3, 1),
+                                                # few rows per token: 8, 4 and 2 tokens share a workgroup; odd S
+                                                (1, 3, 3, 0, 1, 2, 1), (3, 5, 3, 1, 1, 6, 1), (1, 7, 3, 0, 1, 8, 4)])
 def test_prologue_parity(dev, T, H, W, sp, dn, Hq, Hkv):
     S, D = T * H * W, 128
     qr, kr, vr, (gq, bq, gk, bk) = _inputs(S, Hq, Hkv, seed=S + Hq)

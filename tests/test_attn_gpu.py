@@ -407,3 +407,42 @@ def test_repeated_launches_are_bit_identical(dev):
         again8, _ = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L)
         assert torch.equal(again, first) and torch.equal(lse, lse0) and torch.equal(again8, first8)
         del noise
+
+
+def test_graph_capture_and_replay(dev):
+    """The library allocates nothing, never synchronises and launches on the caller's stream, so a prologue +
+    attention pair can be captured into a HIP graph (the reference's enable_cuda_graph case).  Every replay, with
+    new inputs copied into the static buffers and eager work in between, must equal the eager result bit for bit."""
+    S, Hq, Hkv, D, L = 3 * 96, 6, 2, 128, 96
+    g = torch.Generator().manual_seed(11)
+    mk = lambda *shape: torch.randn(*shape, generator=g).bfloat16().to(dev)
+    q_raw, k_raw, v_raw = mk(S, Hq * D), mk(S, Hkv * D), mk(S, Hkv * D)
+    rope = torch.randn(S, 96, generator=g).to(dev)
+    z = torch.zeros(D, device=dev)
+    q = torch.empty(S, Hq, D, dtype=torch.bfloat16, device=dev)
+    kv = torch.empty(S, Hkv, 2 * D, dtype=torch.bfloat16, device=dev)
+    out = torch.empty(S, Hq, D, dtype=torch.bfloat16, device=dev)
+    tq, tk = _ranges(dev, O.q_ranges_for(3, L), O.default_kvrange(0, 3, L))
+
+    def step(dst):
+        M.qk_prologue(q_raw, k_raw, v_raw, rope, z, z, z, z, Hq=Hq, Hkv=Hkv, kv_out=kv, n_cache_rows=S, q_out=q)
+        M.range_attention(q, kv[..., :D], kv[..., D:], tq, tk, L, out=dst, return_lse=False)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step(out)  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step(out)
+    for rep in range(4):
+        for t in (q_raw, k_raw, v_raw):
+            t.copy_(torch.randn(t.shape, generator=g).bfloat16())
+        eager = torch.empty_like(out)
+        step(eager)
+        torch.cuda.synchronize()
+        out.fill_(7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay {rep}"

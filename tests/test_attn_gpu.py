@@ -446,3 +446,38 @@ def test_graph_capture_and_replay(dev):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager), f"replay {rep}"
+
+
+def test_token_strides_beyond_32_bit_tile_offsets(dev):
+    """K / V rows 30 MB apart: a 64-row tile no longer fits the 32-bit offsets of the buffer-addressed tile loads,
+    so the kernels fall back to 64-bit addresses per lane.  Same bits as with packed rows, bf16 and fp8."""
+    Tq, Tk, Hq, Hkv, D = 100, 150, 4, 2, 128
+    stride = 15_000_064  # elements per token; x 2 bytes x (64 + 8) rows > 2^31
+    q, k, v = O.synthetic_qkv(Tq, Tk, Hq, Hkv, D, seed=321)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    tq, tk = _ranges(dev, [[0, 60], [60, 100]], [[0, 150], [17, 90]])
+    base, _ = M.range_attention(qd, kd, vd, tq, tk, 60, return_lse=False)
+    _cmp(base, O.range_attention(q, k, v, [[0, 60], [60, 100]], [[0, 150], [17, 90]]), "packed rows")
+    big_k = torch.empty(Tk * stride, dtype=torch.bfloat16, device=dev)
+    big_v = torch.empty(Tk * stride, dtype=torch.bfloat16, device=dev)
+    ks = big_k.as_strided((Tk, Hkv, D), (stride, D, 1))
+    vs = big_v.as_strided((Tk, Hkv, D), (stride, D, 1))
+    ks.copy_(kd)
+    vs.copy_(vd)
+    far, _ = M.range_attention(qd, ks, vs, tq, tk, 60, return_lse=False)
+    assert torch.equal(far, base)
+    del big_k, big_v, ks, vs
+    # fp8: one byte per element, so twice the element stride
+    q8, qs = M.quantize_fp8(qd, 64)
+    k8, ksc = M.quantize_fp8(kd, 64)
+    v8, vsc = M.quantize_fp8(vd, 64)
+    kw = dict(q_scale=qs, k_scale=ksc, v_scale=vsc, scale_chunk_tokens=64, return_lse=False)
+    base8, _ = M.range_attention(q8, k8, v8, tq, tk, 60, **kw)
+    big_k = torch.empty(Tk * 2 * stride, dtype=torch.float8_e4m3fn, device=dev)
+    big_v = torch.empty(Tk * 2 * stride, dtype=torch.float8_e4m3fn, device=dev)
+    ks = big_k.as_strided((Tk, Hkv, D), (2 * stride, D, 1))
+    vs = big_v.as_strided((Tk, Hkv, D), (2 * stride, D, 1))
+    ks.view(torch.uint8).copy_(k8.view(torch.uint8))
+    vs.view(torch.uint8).copy_(v8.view(torch.uint8))
+    far8, _ = M.range_attention(q8, ks, vs, tq, tk, 60, **kw)
+    assert torch.equal(far8, base8)

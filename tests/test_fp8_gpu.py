@@ -261,3 +261,31 @@ def test_fp8_randomised_ranges_chunks_and_splits(dev):
         # P is rounded to e4m3 (relative error <= 2^-4 per weight); with few keys nothing averages out, so the bound
         # relative to max|ref| is 2^-4 (MAGI_TEST_SWEEP_CASES=400 stays below it; case 88 reaches 4.2e-2)
         assert rel <= 2 ** -4, f"case {case}: {rel}"
+
+
+def test_fp8_many_segments_with_empty_ones(dev):
+    """300 cu_seqlens segments (more than the in-kernel longest-first ranking handles), some without keys, scale
+    chunks of 64 tokens cutting through the segments: against the oracle on the dequantised inputs; empty segments
+    give zero rows."""
+    rng = np.random.default_rng(13)
+    n, C = 300, 64
+    ql = rng.integers(1, 40, size=n)
+    kl = rng.integers(0, 150, size=n)
+    kl[::17] = 0
+    cu_q = np.concatenate([[0], np.cumsum(ql)]).astype(np.int32)
+    cu_k = np.concatenate([[0], np.cumsum(kl)]).astype(np.int32)
+    Hq, Hkv = 4, 2
+    q, k, v = O.synthetic_qkv(int(cu_q[-1]), int(cu_k[-1]), Hq, Hkv, 128, seed=41)
+    q8, qs = M.quantize_fp8(q.to(dev), C)
+    k8, ks = M.quantize_fp8(k.to(dev), C)
+    v8, vs = M.quantize_fp8(v.to(dev), C)
+    out, _ = M.range_attention(q8, k8, v8, torch.tensor(cu_q, device=dev), torch.tensor(cu_k, device=dev), int(ql.max()),
+                               int(kl.max()), ranges_mode=M.MAGI_RANGES_CU, q_scale=qs, k_scale=ks, v_scale=vs,
+                               scale_chunk_tokens=C, return_lse=False)
+    ref = O.varlen_cross_attention(O.dequantize_per_head_chunk(q8.cpu(), qs.cpu(), C),
+                                   O.dequantize_per_head_chunk(k8.cpu(), ks.cpu(), C),
+                                   O.dequantize_per_head_chunk(v8.cpu(), vs.cpu(), C), cu_q, cu_k)
+    rel = ((out.double().cpu() - ref.double()).abs().max() / ref.abs().max()).item()
+    assert torch.isfinite(out).all() and rel <= 2 ** -4, rel
+    empty_rows = np.concatenate([np.arange(cu_q[i], cu_q[i + 1]) for i in range(n) if kl[i] == 0])
+    assert torch.count_nonzero(out[torch.tensor(empty_rows, device=dev)]).item() == 0

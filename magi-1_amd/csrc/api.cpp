@@ -27,6 +27,19 @@ int hip_fail(hipError_t e, const char* what) {
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// compute units of the current device (asked once per device; 256 when the query fails)
+int compute_units() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cached[dev] = n;
+  }
+  return cached[dev];
+}
+
 }  // namespace
 
 extern "C" {
@@ -105,9 +118,19 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.k_split = k_split;
   a.n_ranges = p->n_ranges;
   a.ranges_mode = p->ranges_mode;
+  // q rows per workgroup.  bf16: 384 (12 waves, one workgroup per CU, every K / V tile fetched once for three
+  // times as many rows and one barrier per tile) pays on grids of many rounds with long key ranges; its coarser
+  // q tiles and longer jobs cost more than that on small grids and on short key ranges (cross attention), which
+  // keep 128 (4 waves, three workgroups per CU).
   a.block_m = 128;
-  if (const char* e = std::getenv("MAGI_ATTN_BLOCK_M")) {  // tuning knob: 128 or 256
-    if (std::atoi(e) == 256) a.block_m = 256;
+  if (p->dtype == MAGI_DTYPE_BF16) {
+    const double wg384 = (double)p->Hq * p->n_ranges * ((p->max_seqlen_q + 383) / 384);
+    const bool long_keys = p->max_seqlen_k == 0 || p->max_seqlen_k >= 4096;  // (0 = not stated)
+    if (wg384 >= 24.0 * compute_units() && long_keys) a.block_m = 384;
+    if (const char* e = std::getenv("MAGI_ATTN_BLOCK_M")) {  // tuning knob: 128, 256 or 384
+      const int v = std::atoi(e);
+      if (v == 128 || v == 256 || v == 384) a.block_m = v;
+    }
   }
   if (const char* e = std::getenv("MAGI_ATTN_VARIANT")) a.variant = std::atoi(e);  // tuning knob
   a.tiles_per_range = (p->max_seqlen_q + a.block_m - 1) / a.block_m;

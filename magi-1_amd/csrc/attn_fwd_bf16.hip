@@ -19,12 +19,20 @@
 //
 // A single wavefront cannot keep the MFMA pipe busy (in-order issue, ~5 cycles between its VALU
 // instructions, LDS and MFMA latencies in series): throughput comes from several waves per SIMD
-// in different phases.  The default instantiation runs 3 waves / SIMD: <= 168 VGPRs (shallow
-// operand prefetch) and 48 KB of LDS per workgroup (64-key tiles, K double buffered, ONE V slot that
-// is refilled under the score MFMAs and the softmax of the same tile).  Instantiations with 2 waves
-// / SIMD (deep prefetch, K and V double buffered), with 32-key tiles, and a software-pipelined loop
-// (PIPE: score MFMAs of the next tile, softmax and PV MFMAs of the current one interleaved in one
-// basic block, 2 waves / SIMD) are kept for comparison; on the 720p layer none is faster.
+// in different phases.  Both instantiations that the library picks run 3 waves / SIMD (<= 168 VGPRs,
+// shallow operand prefetch):
+//   * 4 waves per workgroup, three workgroups per CU, 48 KB of LDS each (64-key tiles, K double
+//     buffered, ONE V slot that is refilled under the score MFMAs and the softmax of the same tile,
+//     two barriers per tile): small grids and short key ranges;
+//   * 12 waves per workgroup (DB), ONE workgroup per CU, 64 KB of LDS (K and V double buffered in
+//     four statically named slots, one barrier per tile): every K / V tile is fetched from L2 once
+//     for 384 query rows instead of 128.  On grids of many rounds with long key ranges this is the
+//     faster one, although it needs more cycles: the part is power limited, and the bytes it does
+//     not move come back as clock.
+// Instantiations with 2 waves / SIMD (deep prefetch, K and V double buffered), with 32-key tiles,
+// with 8-wave workgroups, and a software-pipelined loop (PIPE: score MFMAs of the next tile, softmax
+// and PV MFMAs of the current one interleaved in one basic block, 2 waves / SIMD) are kept for
+// comparison; on the 720p layer none is faster.
 //
 // Work decomposition: blockIdx -> (kv head, range slot, q tile, q head within the GQA group),
 // laid out so that the workgroups an XCD receives (blockIdx % 8) share a KV head and walk the
@@ -94,22 +102,26 @@ __device__ __forceinline__ float pair_sum(unsigned pk, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), one, acc, false);
 }
 
-template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool PIPE = false>
+template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool PIPE = false, bool DB = false>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
   constexpr int BM = 32 * NW;
   constexpr int TILE_BYTES = BN * ROW_BYTES;
-  constexpr int LOADS = BN / (4 * NW);     // direct loads per wave per matrix per tile (4 rows each)
+  constexpr int LW = NW > 8 ? 8 : NW;      // waves that load tiles (a 64-row tile is 16 loads of 4 rows)
+  constexpr int LOADS = BN / (4 * LW);     // direct loads per loading wave per matrix per tile (4 rows each)
+  constexpr int WPS = NW * OCC / 4;        // waves per SIMD
   constexpr int TILE_LOADS = 2 * LOADS;    // ... per wave per tile
   constexpr int NT = BN / 32;              // 32-key score tiles per key tile
   constexpr int NS = BN / 16;              // 16-key slabs per key tile
-  constexpr int DK = OCC >= 3 ? 4 : 8;     // K operands in flight
-  constexpr int DV = OCC >= 3 ? 4 : 8;     // V operands in flight
+  constexpr int DK = WPS >= 3 ? 4 : 8;     // K operands in flight
+  constexpr int DV = WPS >= 3 ? 4 : 8;     // V operands in flight
+  constexpr bool VEARLY = !VSINGLE && WPS < 3;  // first V operands fetched under the last score MFMAs (needs registers)
   static_assert(LOADS >= 1 && NSTAGE >= 2 && NSTAGE <= 4, "bad tile configuration");
   static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");
   static_assert(!PIPE || (NSTAGE == 2 && BN == 64 && !VSINGLE), "pipelined loop: 64-key tiles, two K slots and two V slots");
+  static_assert(!DB || (NSTAGE == 2 && !VSINGLE && !PIPE), "static double buffer: two K slots and two V slots");
   // ring of NSTAGE (K tile, V tile) pairs, or in single-V mode K slot 0, K slot 1, V slot
   // (the pipelined loop declares its four slots as separate objects instead and leaves this one a stub)
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[PIPE ? 1 : VSINGLE ? 3 : 2 * NSTAGE][PIPE ? 16 : TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[(PIPE || DB) ? 1 : VSINGLE ? 3 : 2 * NSTAGE][(PIPE || DB) ? 16 : TILE_BYTES];
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -197,6 +209,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
   // LOADS load instructions per wave per matrix per tile, always, so outstanding loads can be counted.
   auto issue_mat = [&](int k0, unsigned char* tile_base, bool is_v) {
+    if (NW > LW && w >= LW) return;  // (wave uniform) the other waves only consume
     unsigned char* dst = tile_base + w * 1024;
     const long st = is_v ? vs_t : ks_t;
     const char* colp = is_v ? vcolp : kcolp;
@@ -212,8 +225,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       const unsigned voff = is_v ? vvoff : kvoff;
 #pragma unroll
       for (int j = 0; j < LOADS; ++j)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * NW * 1024), 16, voff,
-                                                 (int)((unsigned)(4 * NW * j) * (unsigned)st), 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * LW * 1024), 16, voff,
+                                                 (int)((unsigned)(4 * LW * j) * (unsigned)st), 0, 0);
     } else {  // ragged end of the range, or a tile that straddles the two key segments
       // (rare: the lane geometry is re-derived here from an opaque copy of the lane index, so that nothing of
       // it occupies registers across the main loop)
@@ -224,9 +237,9 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       const int chunk = is_v ? (slot_s ^ (lrow_s << 2)) : (slot_s ^ ((4 * (w & 3) + lrow_s) & 15));
 #pragma unroll
       for (int j = 0; j < LOADS; ++j) {
-        const int row = min(k0 + row_in_tile0 + 4 * NW * j, ke - 1);
+        const int row = min(k0 + row_in_tile0 + 4 * LW * j, ke - 1);
         const char* p = colp + (long)row * st + (row >= k_split ? d2 : 0) + chunk * 16;
-        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(p), LDS_PTR(void, dst + j * NW * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(GLOBAL_PTR(p), LDS_PTR(void, dst + j * LW * 1024), 16, 0, 0);
       }
     }
   };
@@ -433,45 +446,9 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       step(it + 1, odd, sB, sA);
     }
   } else {
-  if (VSINGLE) {
-    issue_mat(ks, &smem[0][0], false);
-  } else {
-#pragma unroll
-    for (int p = 0; p < NSTAGE - 1; ++p)
-      if (p < n_tiles) issue_tile(ks + p * BN, p);
-  }
-  int stage = 0;
-  for (int it = 0; it < n_tiles; ++it) {
-    const int k0 = ks + it * BN;
-    if (VSINGLE) {
-      // single-V mode (48 KB of LDS, three workgroups per CU): K(it) was requested one iteration ago; V(it)
-      // is requested now, into the one V slot that PV(it-1) has just released, and lands under the score
-      // MFMAs and the softmax of this tile; a second barrier publishes it before PV(it).
-      wait_vmcnt<0>();
-      __syncthreads();
-      issue_mat(k0, &smem[2][0], true);
-      if (it + 1 < n_tiles) issue_mat(k0 + BN, &smem[(it + 1) & 1][0], false);
-    } else {
-      // tile `it` must have landed; up to NSTAGE-2 younger tiles may still be in flight
-      const int younger = min(NSTAGE - 2, n_tiles - 1 - it);
-      if (NSTAGE >= 4 && younger == 2)
-        wait_vmcnt<2 * TILE_LOADS>();
-      else if (NSTAGE >= 3 && younger == 1)
-        wait_vmcnt<TILE_LOADS>();
-      else
-        wait_vmcnt<0>();
-      __syncthreads();  // everybody's share landed; the stage read in the previous iteration is free again
-      if (it + NSTAGE - 1 < n_tiles) {
-        int st = stage + NSTAGE - 1;
-        if (st >= NSTAGE) st -= NSTAGE;
-        issue_tile(k0 + (NSTAGE - 1) * BN, st);
-      }
-    }
-    const unsigned char* Kt = &smem[VSINGLE ? (it & 1) : 2 * stage][0];
-    const unsigned char* Vt = &smem[VSINGLE ? 2 : 2 * stage + 1][0];
-    stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
-    if (!VSINGLE && !wave_on) continue;
-
+  // One key tile for this wave: scores, online softmax, PV.  Kt / Vt: the tile's K and V slots; before_pv runs
+  // between the softmax and the first V operand read (the single-V mode publishes V(it) there).
+  auto compute_tile = [&](const unsigned char* Kt, const unsigned char* Vt, int k0, auto before_pv) {
     // LDS operand fetchers
     auto read_k = [&](int idx) -> bf16x8 {  // idx = 8t + kk
       return *LDS_PTR(const bf16x8, Kt + ((base_k ^ ((idx & 7) << 5)) + (idx >> 3) * 32 * ROW_BYTES));
@@ -500,7 +477,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kbuf[idx % DK], qf[kk], kk == 0 ? zero16 : s_acc[t], 0, 0, 0);
       if (idx + DK < RK)
         kbuf[idx % DK] = read_k(idx + DK);
-      else if (!VSINGLE && idx + DK - RK < DV)
+      else if (VEARLY && idx + DK - RK < DV)
         vbuf[idx + DK - RK] = read_v(idx + DK - RK);
       if (DK == 8 && NT == 2 && idx == 7) __builtin_amdgcn_sched_barrier(0);
     }
@@ -554,12 +531,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
     // O^T[d][q] += V^T[d][key] P^T[key][q]; V operands run DV reads ahead
     __builtin_amdgcn_sched_barrier(0);
-    if (VSINGLE) {
-      if (it + 1 < n_tiles)
-        wait_vmcnt<LOADS>();  // V(it) landed; the K(it+1) loads issued after it may still be in flight
-      else
-        wait_vmcnt<0>();
-      __syncthreads();
+    before_pv();
+    if (!VEARLY) {
 #pragma unroll
       for (int p = 0; p < DV; ++p) vbuf[p] = read_v(p);
     }
@@ -569,7 +542,85 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       o_acc[mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vbuf[p % DV], p_operand(s), o_acc[mb], 0, 0, 0);
       if (p + DV < RV) vbuf[p % DV] = read_v(p + DV);
     }
+  };
+  if constexpr (DB) {
+    // K and V double buffered in four separate LDS objects, the loop unrolled by two so that every slot is named
+    // statically (an operand read then never waits for the direct loads in flight to the other pair of slots);
+    // one barrier per tile, and the loads of tile it+1 have the whole of iteration it to land.
+    __shared__ __attribute__((aligned(1024))) unsigned char dK0[TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char dV0[TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char dK1[TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char dV1[TILE_BYTES];
+    issue_mat(ks, dK0, false);
+    issue_mat(ks, dV0, true);
+    auto step = [&](int it, auto bc) {
+      constexpr int B = decltype(bc)::value;
+      const int k0 = ks + it * BN;
+      wait_vmcnt<0>();
+      __syncthreads();
+      if (it + 1 < n_tiles) {
+        issue_mat(k0 + BN, B ? dK0 : dK1, false);
+        issue_mat(k0 + BN, B ? dV0 : dV1, true);
+      }
+      if (!wave_on) return;
+      compute_tile(B ? dK1 : dK0, B ? dV1 : dV0, k0, []() {});
+    };
+    for (int it = 0; it < n_tiles; it += 2) {
+      step(it, std::integral_constant<int, 0>{});
+      if (it + 1 >= n_tiles) break;
+      step(it + 1, std::integral_constant<int, 1>{});
+    }
+  } else {
+  if (VSINGLE) {
+    issue_mat(ks, &smem[0][0], false);
+  } else {
+#pragma unroll
+    for (int p = 0; p < NSTAGE - 1; ++p)
+      if (p < n_tiles) issue_tile(ks + p * BN, p);
   }
+  int stage = 0;
+  for (int it = 0; it < n_tiles; ++it) {
+    const int k0 = ks + it * BN;
+    if (VSINGLE) {
+      // single-V mode (48 KB of LDS, three workgroups per CU): K(it) was requested one iteration ago; V(it)
+      // is requested now, into the one V slot that PV(it-1) has just released, and lands under the score
+      // MFMAs and the softmax of this tile; a second barrier publishes it before PV(it).
+      wait_vmcnt<0>();
+      __syncthreads();
+      issue_mat(k0, &smem[2][0], true);
+      if (it + 1 < n_tiles) issue_mat(k0 + BN, &smem[(it + 1) & 1][0], false);
+    } else {
+      // tile `it` must have landed; up to NSTAGE-2 younger tiles may still be in flight
+      const int younger = min(NSTAGE - 2, n_tiles - 1 - it);
+      if (NSTAGE >= 4 && younger == 2)
+        wait_vmcnt<2 * TILE_LOADS>();
+      else if (NSTAGE >= 3 && younger == 1)
+        wait_vmcnt<TILE_LOADS>();
+      else
+        wait_vmcnt<0>();
+      __syncthreads();  // everybody's share landed; the stage read in the previous iteration is free again
+      if (it + NSTAGE - 1 < n_tiles) {
+        int st = stage + NSTAGE - 1;
+        if (st >= NSTAGE) st -= NSTAGE;
+        issue_tile(k0 + (NSTAGE - 1) * BN, st);
+      }
+    }
+    const unsigned char* Kt = &smem[VSINGLE ? (it & 1) : 2 * stage][0];
+    const unsigned char* Vt = &smem[VSINGLE ? 2 : 2 * stage + 1][0];
+    stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
+    if (!VSINGLE && !wave_on) continue;
+
+    compute_tile(Kt, Vt, k0, [&]() {
+      if (VSINGLE) {
+        if (it + 1 < n_tiles)
+          wait_vmcnt<LOADS>();  // V(it) landed; the K(it+1) loads issued after it may still be in flight
+        else
+          wait_vmcnt<0>();
+        __syncthreads();
+      }
+    });
+  }
+  }  // !DB
   }  // !PIPE
 
   if (!wave_on) return;
@@ -597,7 +648,9 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  if (a.block_m == 256 && a.variant == 3)  // software-pipelined loop, 8 waves, 256 query rows, 2 waves / SIMD
+  if (a.block_m == 384)  // 12 waves, 384 query rows, one workgroup per CU = 3 waves / SIMD sharing every tile
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true>), dim3(grid), dim3(768), 0, stream, a);
+  else if (a.block_m == 256 && a.variant == 3)  // software-pipelined loop, 8 waves, 256 query rows, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false, true>), dim3(grid), dim3(512), 0, stream, a);
   else if (a.block_m == 256)  // 8 waves, 256 query rows, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false>), dim3(grid), dim3(512), 0, stream, a);

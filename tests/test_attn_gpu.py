@@ -481,3 +481,31 @@ def test_token_strides_beyond_32_bit_tile_offsets(dev):
     vs.view(torch.uint8).copy_(v8.view(torch.uint8))
     far8, _ = M.range_attention(q8, ks, vs, tq, tk, 60, **kw)
     assert torch.equal(far8, base8)
+
+
+@pytest.mark.parametrize("block_m", ["384", "256", "128"])
+def test_every_workgroup_shape_on_the_small_cases(dev, monkeypatch, block_m):
+    """The library picks 384-row (12-wave) workgroups for grids of many rounds and 128-row ones otherwise, so the
+    small parity cases would only ever meet the latter: force each shape (a tuning knob of the library) through
+    the chunk-causal cases, a sliding window in shuffled order, the two-segment key axis and a strided cache."""
+    monkeypatch.setenv("MAGI_ATTN_BLOCK_M", block_m)
+    for L, dn, sp, Hq, Hkv in CASES:
+        q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=4321 + L)
+        qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+        tq, tk = _ranges(dev, qr, kr)
+        out, lse = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L)
+        _cmp(out, O.range_attention(q, k, v, qr, kr), f"block_m={block_m} L={L}")
+        assert (lse.cpu() - O.range_attention_lse(q, k, v, qr, kr)).abs().max() < 5e-3
+    L, dn, sp, Hq, Hkv = 500, 4, 3, 6, 2
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=77)
+    qr = O.q_ranges_for(dn, L)[[2, 0, 3, 1]]
+    kr = O.noise2clean_kvrange(sp, dn, L, [5, 4, 3, 2], 1, [32, 20, 9, 0], 32)[[2, 0, 3, 1]]
+    ref = O.range_attention(q, k, v, qr, kr)
+    tq, tk = _ranges(dev, qr, kr)
+    cache = torch.cat([k, v], dim=-1).to(dev)  # interleaved [T, Hkv, 2D]: strided K and V views
+    out, _ = M.range_attention(q.to(dev), cache[..., :128], cache[..., 128:], tq, tk, L, return_lse=False)
+    _cmp(out, ref, f"block_m={block_m} window, strided cache")
+    split = 3 * L + 123
+    out2, _ = M.range_attention(q.to(dev), cache[:split, :, :128], cache[:split, :, 128:], tq, tk, L,
+                                k2=cache[split:, :, :128], v2=cache[split:, :, 128:], k_split=split, return_lse=False)
+    _cmp(out2, ref, f"block_m={block_m} two segments")

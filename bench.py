@@ -12,6 +12,7 @@ timings of that kernel alone, and `cpu_baseline` times the CPU oracle (torch SDP
 ranges) on a bounded sample of the same workload on this machine's host cores.
 """
 import argparse
+import math
 import json
 import os
 import sys
@@ -27,6 +28,7 @@ import torch
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_FP8_TFLOPS = 5000.0
 PEAK_HBM_GBS = 8000.0
+Q_PREMUL = 128 ** -0.5 * math.log2(math.e)  # softmax_scale * log2(e) at head_dim 128
 # HBM-side bytes per launch on the 720p workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # plain copy of known size in the same run (FETCH_SIZE x2.0, WRITE_SIZE x1.0): profiles/bench_720p_hbm_traffic_pmc.txt
 MEASURED_TRAFFIC = {"720p-24B": {"core": 186.8e9 + 1.09e9, "prologue": 1.449e9 + 1.434e9}}
@@ -111,13 +113,15 @@ def run_step(inp, ev=None):
         if ev is not None:
             ev[key][which].record()
 
+    # as the layer module does: the prologue folds softmax_scale * log2(e) into q ahead of q's rounding to bf16
+    # and the attention call says so (the kernel then has no per-score multiply)
     rec("prologue", 0)
     M.qk_prologue(inp["q_raw"], inp["k_raw"], inp["v_raw"], inp["rope"], z, z, z, z, Hq=inp["Hq"], Hkv=inp["Hkv"],
-                  kv_out=cache[sp * L:], n_cache_rows=inp["S"], q_out=inp["q"])
+                  kv_out=cache[sp * L:], n_cache_rows=inp["S"], q_out=inp["q"], q_premul=Q_PREMUL)
     rec("prologue", 1)
     rec("core", 0)
     M.range_attention(inp["q"], cache[..., :D], cache[..., D:], inp["q_ranges"], inp["k_ranges"], L,
-                      out=inp["out"], return_lse=False)
+                      out=inp["out"], return_lse=False, q_prescaled=True)
     rec("core", 1)
     rec("cross", 0)
     qx = M.head_norm(inp["qx_raw"], z, z)
@@ -139,7 +143,8 @@ def fp8_leg(inp, core_fl, bf16_tflops, steps):
     cache = inp["cache"]
     # power-of-two scales, softmax_scale * log2(e) folded into q before quantisation: the scales ride on the
     # MFMA's block-scale operands and the kernel does no per-score multiply
-    q8, qs = M.quantize_fp8(inp["q"], L, premul=D ** -0.5 * math.log2(math.e), pow2_scales=True)
+    # (inp["q"] already carries that factor from the prologue)
+    q8, qs = M.quantize_fp8(inp["q"], L, premul=1.0, pow2_scales=True)
     k8, ks = M.quantize_fp8(cache[..., :D], L, pow2_scales=True)
     v8, vs = M.quantize_fp8(cache[..., D:], L, pow2_scales=True)
     out8 = torch.empty_like(inp["out"])
@@ -180,7 +185,7 @@ def cpu_baseline(inp, rows_per_chunk=6144):
     fl = O.attention_flops(qr, kr, G, D)
     torch.set_num_threads(os.cpu_count() if os.cpu_count() and os.cpu_count() <= 64 else torch.get_num_threads())
     t0 = time.perf_counter()
-    o = O.range_attention(q, k, v, qr, kr)
+    o = O.range_attention(q, k, v, qr, kr, softmax_scale=math.log(2.0))  # q carries softmax_scale * log2(e)
     dt = time.perf_counter() - t0
     return dict(value=fl / dt / 1e12, unit="TFLOP/s", cores=torch.get_num_threads(), kind="port",
                 sample=f"first {rows} q rows of each of the {dn} chunks x {G} q heads of kv head 0, full key ranges, "

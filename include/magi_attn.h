@@ -35,6 +35,11 @@ extern "C" {
  * scales then ride on the MFMA's block-scale operands and the kernel does no per-score multiply;
  * softmax_scale is ignored. */
 #define MAGI_ATTN_FP8_POW2_PRESCALED 1
+/* bf16 path: q already carries softmax_scale * log2(e) (magi_qk_prologue with q_premul set to it multiplies before
+ * its one rounding to bf16, so nothing is lost), i.e. the scores q.k are exp2 exponents.  The kernel then skips the
+ * per-score multiply and, where it has an instantiation for it, lets the score MFMAs accumulate onto the negated
+ * running maximum; softmax_scale is ignored.  No counterpart in the reference, whose kernels take unscaled q. */
+#define MAGI_ATTN_Q_PRESCALED 2
 
 #define MAGI_RANGES_PAIRS 0 /* int32 [n, 2]: range i = [r[2i], r[2i+1])          */
 #define MAGI_RANGES_CU 1    /* int32 [n + 1] cumulative: range i = [r[i], r[i+1]) */
@@ -129,6 +134,8 @@ int magi_attn_fwd(const magi_attn_args* args, void* stream);
  *       rotary_dim = 2*R2 <= D; NULL disables rotary
  * gq,bq,gk,bk  fp32 [D] norm parameters (gamma stored zero-centred); b* may be NULL
  * q_out [S, Hq, D] bf16 contiguous
+ * q_premul  factor applied to q after norm and rotary, before the rounding to bf16 (0 = none, like 1); set it to
+ *         softmax_scale * log2(e) when the attention call passes MAGI_ATTN_Q_PRESCALED
  * kv_out  row 0 of the destination for the first n_cache_rows tokens: [*, Hkv, 2D] with token
  *         stride kv_stride_t; K goes to [..., 0:D], V to [..., D:2D]
  * kv_tail destination of tokens >= n_cache_rows (same layout, row index t - n_cache_rows); may be
@@ -153,7 +160,7 @@ typedef struct magi_prologue_args {
   int32_t norm_kind;
   float eps;
   int32_t batch; /* tokens are ordered (position, batch): rope row of token t is t / batch; 0 or 1 = no batch */
-  int32_t reserved;
+  float q_premul;
 } magi_prologue_args;
 
 int magi_qk_prologue(const magi_prologue_args* args, void* stream);

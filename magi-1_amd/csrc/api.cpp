@@ -145,6 +145,7 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.per_xcd = (a.total_wgs + 7u) / 8u;
   const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 1.0f / std::sqrt((float)p->D);
   a.scale_log2 = scale * 1.4426950408889634f;
+  if (p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)) a.scale_log2 = 1.f;  // q . k is the exp2 exponent
 
   hipError_t e = p->dtype == MAGI_DTYPE_BF16 ? magi::launch_attn_fwd_bf16(a, static_cast<hipStream_t>(stream))
                                              : magi::launch_attn_fwd_fp8(a, static_cast<hipStream_t>(stream));
@@ -205,6 +206,9 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   a.norm_kind = p->norm_kind;
   a.eps = p->eps;
   a.batch = p->batch > 1 ? p->batch : 1;
+  if (!(p->q_premul == p->q_premul) || std::fabs(p->q_premul) > 1e30f)
+    return fail(MAGI_EINVAL, "magi_qk_prologue: q_premul is not finite");
+  a.q_premul = p->q_premul == 0.f ? 1.f : p->q_premul;
   hipError_t e = magi::launch_prologue(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_qk_prologue launch");
   return MAGI_OK;

@@ -102,7 +102,7 @@ __device__ __forceinline__ float pair_sum(unsigned pk, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), one, acc, false);
 }
 
-template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool PIPE = false, bool DB = false>
+template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool PIPE = false, bool DB = false, bool PRESC = false>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
   constexpr int BM = 32 * NW;
   constexpr int TILE_BYTES = BN * ROW_BYTES;
@@ -112,8 +112,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   constexpr int TILE_LOADS = 2 * LOADS;    // ... per wave per tile
   constexpr int NT = BN / 32;              // 32-key score tiles per key tile
   constexpr int NS = BN / 16;              // 16-key slabs per key tile
-  constexpr int DK = WPS >= 3 ? 4 : 8;     // K operands in flight
-  constexpr int DV = WPS >= 3 ? 4 : 8;     // V operands in flight
+  constexpr int DK = PRESC ? 2 : WPS >= 3 ? 4 : 8;  // K operands in flight
+  constexpr int DV = PRESC ? 2 : WPS >= 3 ? 4 : 8;  // V operands in flight
   constexpr bool VEARLY = !VSINGLE && WPS < 3;  // first V operands fetched under the last score MFMAs (needs registers)
   static_assert(LOADS >= 1 && NSTAGE >= 2 && NSTAGE <= 4, "bad tile configuration");
   static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");
@@ -190,6 +190,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
     const char* qp = a.q + (long)qr * a.qs_t + (long)h * a.qs_h + g * 16;
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) qf[kk] = *(const bf16x8*)(qp + kk * 32);
+
   }
 
   // ---- K/V tile loader: wave w fills rows 4*(w + NW*j) .. +3; lane l sits at row +(l >> 4), slot l & 15 ----
@@ -222,7 +223,16 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       // over a hundred cycles per instruction.
       const char* b = colp + (long)k0 * st + (k0 >= k_split ? d2 : 0);
       const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)b, 0, 0x7fffffff, 0x00020000);
-      const unsigned voff = is_v ? vvoff : kvoff;
+      unsigned voff = is_v ? vvoff : kvoff;
+      if constexpr (PRESC) {
+        // (this instantiation has no registers to spare: the lane offset is re-derived from an opaque copy of
+        // the lane index instead of living across the loop)
+        int lane = l;
+        asm volatile("" : "+v"(lane));
+        const int lr = lane >> 4, sl = lane & 15;
+        const int chunk = is_v ? (sl ^ (lr << 2)) : (sl ^ ((4 * (w & 3) + lr) & 15));
+        voff = (unsigned)(4 * w + lr) * (unsigned)st + (unsigned)(chunk * 16);
+      }
 #pragma unroll
       for (int j = 0; j < LOADS; ++j)
         __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * LW * 1024), 16, voff,
@@ -261,7 +271,14 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
     for (int v = 0; v < 16; ++v) o_acc[mb][v] = 0.f;
-  float m_run = -__builtin_inff();  // running max of raw scores
+  // running max of the raw scores.  PRESC (q carries softmax_scale * log2(e), so the scores are exp2 exponents): the
+  // score MFMAs accumulate onto neg_m = -(running max) in all 16 registers (a lane's registers all belong to one
+  // query) and deliver exponent - max directly: no per-score multiply-subtract; the maximum starts at 0
+  float m_run = PRESC ? 0.f : -__builtin_inff();
+  f32x16 neg_m;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) neg_m[v] = 0.f;
+  bool first = true;
   float l_run = 0.f;                // this lane's share of the running sum
   const float c = a.scale_log2;
   const bool wave_on = (q0 + 32 * w) < qe;
@@ -474,7 +491,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 #pragma unroll
     for (int idx = 0; idx < RK; ++idx) {
       const int t = idx >> 3, kk = idx & 7;
-      s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kbuf[idx % DK], qf[kk], kk == 0 ? zero16 : s_acc[t], 0, 0, 0);
+      s_acc[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kbuf[idx % DK], qf[kk],
+                                                         kk == 0 ? (PRESC ? neg_m : zero16) : s_acc[t], 0, 0, 0);
       if (idx + DK < RK)
         kbuf[idx % DK] = read_k(idx + DK);
       else if (VEARLY && idx + DK - RK < DV)
@@ -498,11 +516,44 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 #pragma unroll
       for (int v = (t == 0 ? 3 : 0); v < 16; v += 2) mx = max3(mx, s_acc[t][v], s_acc[t][v + 1 < 16 ? v + 1 : v]);
     mx = half_swap_max(mx);
+    float psum = 0.f;  // row sum of the probabilities as rounded to bf16, i.e. of what the PV product uses
+    if constexpr (PRESC) {
+      // s_acc holds exponent - m_run: a positive value is a new row maximum (rare after the first tiles)
+      const bool raise = first || mx > 0.f;
+      if (__builtin_amdgcn_ballot_w64(raise) != 0) {
+        const float delta = raise ? mx : 0.f;
+        const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);
+        l_run *= alpha;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) neg_m[v] -= delta;  // (the running maximum is -neg_m)
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+#pragma unroll
+          for (int v = 0; v < 16; ++v) s_acc[t][v] -= delta;
+        if (!first) {
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+        }
+      }
+      first = false;
+#pragma unroll
+      for (int s = 0; s < NS; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+          f32x16& sv = s_acc[s >> 1];
+          const int v0 = 8 * (s & 1) + e;
+          const unsigned pk = pack_bf16x2(__builtin_amdgcn_exp2f(sv[v0]), __builtin_amdgcn_exp2f(sv[v0 + 1]));
+          psum = pair_sum(pk, psum);
+          sv[8 * (s & 1) + (e >> 1)] = __builtin_bit_cast(float, pk);
+        }
+      l_run += psum;
+    } else {
     const float m_new = fmaxf(m_run, mx);
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_new) * c);
     const float mc = m_new * c;
     m_run = m_new;
-    float psum = 0.f;  // row sum of the probabilities as rounded to bf16, i.e. of what the PV product uses
     // the packed probabilities of slab s overwrite the first four of the eight score registers they came from
 #pragma unroll
     for (int s = 0; s < NS; ++s)
@@ -522,6 +573,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
         for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
+    }
     }
     auto p_operand = [&](int s) -> bf16x8 {  // B operand of the PV MFMAs for slab s
       const f32x16& sv = s_acc[s >> 1];
@@ -640,7 +692,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
         *(u32x2*)(op + d * 2) = pk;
       }
     if (a.lse && g == 0)
-      a.lse[(long)h * a.total_q + q_row] = (m_run * c + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
+      a.lse[(long)h * a.total_q + q_row] = ((PRESC ? -neg_m[0] : m_run * c) + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   }
 }
 
@@ -648,7 +700,9 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  if (a.block_m == 384)  // 12 waves, 384 query rows, one workgroup per CU = 3 waves / SIMD sharing every tile
+  if (a.block_m == 384 && (a.flags & 2) && a.variant != 7)  // ... q pre-scaled: scores are exp2 exponents (PRESC)
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true, true>), dim3(grid), dim3(768), 0, stream, a);
+  else if (a.block_m == 384)  // 12 waves, 384 query rows, one workgroup per CU = 3 waves / SIMD sharing every tile
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true>), dim3(grid), dim3(768), 0, stream, a);
   else if (a.block_m == 256 && a.variant == 3)  // software-pipelined loop, 8 waves, 256 query rows, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false, true>), dim3(grid), dim3(512), 0, stream, a);
@@ -660,7 +714,7 @@ hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false>), dim3(grid), dim3(256), 0, stream, a);
   else if (a.variant == 3)  // software-pipelined loop, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false, true>), dim3(grid), dim3(256), 0, stream, a);
-  else  // default: 64-key tiles, double-buffered K, single V slot, 3 waves / SIMD
+  else  // 4 waves, 64-key tiles, double-buffered K, single V slot, three workgroups per CU
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();
 }

@@ -56,6 +56,7 @@ struct PrologueKernArgs {
   int norm_kind;
   float eps;
   int batch;
+  float q_premul;  // factor on q before the bf16 rounding (1 = none)
 };
 hipError_t launch_prologue(const PrologueKernArgs& a, hipStream_t stream);
 

@@ -150,6 +150,10 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
           x[8 + i] = x1 * sn[i] + x2 * cs[i];
         }
       }
+      if (kind == 0 && a.q_premul != 1.f) {  // e.g. softmax_scale * log2(e), ahead of the one rounding to bf16
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x[i] *= a.q_premul;
+      }
       *(u32x4*)(dst + ea * 2) = pack8(x);
       *(u32x4*)(dst + eb * 2) = pack8(x + 8);
     }

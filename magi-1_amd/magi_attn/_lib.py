@@ -19,6 +19,7 @@ MAGI_NORM_LAYERNORM_1P = 0
 MAGI_NORM_RMSNORM_1P = 1
 MAGI_NORM_NONE = 2
 MAGI_ATTN_FP8_POW2_PRESCALED = 1
+MAGI_ATTN_Q_PRESCALED = 2
 
 
 class MagiError(RuntimeError):
@@ -55,7 +56,7 @@ class PrologueArgs(C.Structure):
         ("kv_stride_t", C.c_int64), ("kv_tail_stride_t", C.c_int64),
         ("S", C.c_int32), ("n_cache_rows", C.c_int32),
         ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32), ("R2", C.c_int32),
-        ("norm_kind", C.c_int32), ("eps", C.c_float), ("batch", C.c_int32), ("reserved", C.c_int32),
+        ("norm_kind", C.c_int32), ("eps", C.c_float), ("batch", C.c_int32), ("q_premul", C.c_float),
     ]
 
 

@@ -66,6 +66,7 @@ def range_attention(
     v_scale: Optional[torch.Tensor] = None,
     scale_chunk_tokens: int = 0,
     fp8_pow2_prescaled: bool = False,
+    q_prescaled: bool = False,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = True,
     zero_init: bool = True,
@@ -74,6 +75,9 @@ def range_attention(
 
     k and v may be strided views (e.g. the two halves of an interleaved KV cache); with
     k2 / v2 the key axis is the concatenation [k[:k_split] | k2] without copying.
+
+    q_prescaled (bf16): q already carries softmax_scale * log2(e) (qk_prologue(..., q_premul=that)), so q . k is the
+    exp2 exponent: the kernel skips its per-score multiply; softmax_scale is ignored.
     """
     _check_thd(q, "q")
     _check_thd(k, "k")
@@ -129,7 +133,7 @@ def range_attention(
     a.dtype = _dtype_code(q)
     a.scale_chunk_tokens = int(scale_chunk_tokens)
     a.softmax_scale = 0.0 if softmax_scale is None else float(softmax_scale)
-    a.flags = L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0
+    a.flags = (L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0) | (L.MAGI_ATTN_Q_PRESCALED if q_prescaled else 0)
     with torch.cuda.device(q.device):
         L.check(L.lib().magi_attn_fwd(C.byref(a), _stream()))
     return out, lse
@@ -194,9 +198,12 @@ def apply_rotary_emb(x, cos, sin, interleaved=False, inplace=False, **_unused):
 def qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int, eps: float = 1e-6,
                 norm_kind: int = L.MAGI_NORM_LAYERNORM_1P, kv_out: Optional[torch.Tensor] = None,
                 n_cache_rows: Optional[int] = None, kv_tail: Optional[torch.Tensor] = None,
-                q_out: Optional[torch.Tensor] = None, batch: int = 1):
+                q_out: Optional[torch.Tensor] = None, batch: int = 1, q_premul: float = 1.0):
     """Fused norm + rotary + cast + KV write.  q_raw [S, Hq*D], k_raw / v_raw [S, Hkv*D] bf16 (row
     strided views allowed); rope [S, 2*R2] fp32 (sin | cos) or None.
+
+    q_premul multiplies q after norm and rotary, before the one rounding to bf16 (softmax_scale * log2(e) for
+    range_attention(..., q_prescaled=True)).
 
     kv_out is the destination of the first n_cache_rows tokens (a view of the cache starting
     at the write position, [>= n_cache_rows, Hkv, 2D]); kv_tail takes the rest.  With neither,
@@ -239,6 +246,7 @@ def qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int,
     a.S, a.n_cache_rows = S, int(n_cache_rows)
     a.Hq, a.Hkv, a.D, a.R2 = Hq, Hkv, D, R2
     a.norm_kind, a.eps, a.batch = int(norm_kind), float(eps), int(batch)
+    a.q_premul = float(q_premul)
     with torch.cuda.device(dev):
         L.check(L.lib().magi_qk_prologue(C.byref(a), _stream()))
     return q_out, kv_out, kv_tail

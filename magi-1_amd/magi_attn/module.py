@@ -159,6 +159,9 @@ class FullyParallelAttention(torch.nn.Module):
         if attention_dtype not in ("bf16", "fp8"):
             raise ValueError("attention_dtype must be 'bf16' or 'fp8'")
         self.attention_dtype = attention_dtype
+        # forward() has the prologue fold softmax_scale * log2(e) into q ahead of q's one rounding to bf16 and tells
+        # the attention kernel so (no per-score multiply there); get_q / get_qkv return q unscaled, as the reference
+        self._q_premul = kv_channels ** -0.5 * math.log2(math.e)
         self.layer_number = layer_number
         self.hidden_size_per_attention_head = kv_channels
         self.num_attention_heads = num_attention_heads
@@ -296,8 +299,9 @@ class FullyParallelAttention(torch.nn.Module):
         return q, kv[..., :D].contiguous(), kv[..., D:].contiguous()
 
     def _fused_qkv(self, mixed_qqkv, cos_emb, sin_emb, want_q=True, kv_out=None, n_cache_rows=None, kv_tail=None,
-                   raw=None):
-        """raw: (q_raw, k_raw, v_raw) already projected (views of forward_qkvx's result), else projected here."""
+                   raw=None, q_premul=1.0):
+        """raw: (q_raw, k_raw, v_raw) already projected (views of forward_qkvx's result), else projected here.
+        q_premul: factor folded into q ahead of its rounding to bf16 (see qk_prologue)."""
         sq, b = mixed_qqkv.shape[0], mixed_qqkv.shape[1]
         S = sq * b
         Hq, Hkv = self.num_attention_heads, self.num_query_groups_per_partition
@@ -314,7 +318,8 @@ class FullyParallelAttention(torch.nn.Module):
         gq, bq = self.q_layernorm.gamma_beta_fp32()
         gk, bk = self.k_layernorm.gamma_beta_fp32()
         q, kv, tail = qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, Hq=Hq if want_q else 0, Hkv=Hkv,
-                                  eps=self.eps, kv_out=kv_out, n_cache_rows=n_cache_rows, kv_tail=kv_tail, batch=b)
+                                  eps=self.eps, kv_out=kv_out, n_cache_rows=n_cache_rows, kv_tail=kv_tail, batch=b,
+                                  q_premul=q_premul)
         return (q if want_q else None), (kv if tail is None else (kv, tail))
 
     def get_xqkv(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor, qx_raw: Optional[torch.Tensor] = None):
@@ -354,14 +359,16 @@ class FullyParallelAttention(torch.nn.Module):
         return key_and_value[..., :D].contiguous(), key_and_value[..., D:].contiguous()
 
     def core_attention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, bs: int,
-                       meta_args: ModelMetaArgs, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                       meta_args: ModelMetaArgs, out: Optional[torch.Tensor] = None,
+                       q_prescaled: bool = False) -> torch.Tensor:
         """query [(sq b), Hq, D], key / value [(sk b), Hkv, D] -> [(sq b), Hq, D]; dit_module.py:1023-1066.
         bs > 1 only occurs with one range per batch row (asserted there too).  `out` (bs == 1 only) is a
-        destination view, possibly in the grouped layout of range_attention."""
+        destination view, possibly in the grouped layout of range_attention.  q_prescaled: query carries
+        softmax_scale * log2(e) (see range_attention)."""
         p = meta_args.core_attn_params
         if bs == 1:
             out, _ = range_attention(query, key, value, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                     out=out, return_lse=False)
+                                     out=out, return_lse=False, q_prescaled=q_prescaled)
             return out
         if meta_args.denoising_range_num > 1:
             raise ValueError("bs > 1 with several denoising ranges is not a layout the pipeline produces")
@@ -371,7 +378,7 @@ class FullyParallelAttention(torch.nn.Module):
         kone = torch.tensor([[0, key.shape[0] // bs]], dtype=torch.int32, device=query.device)
         for b in range(bs):  # batch rows are strided views of the (sq b) token axis: no transposes
             range_attention(query[b::bs], key[b::bs], value[b::bs], one, kone, sq, key.shape[0] // bs,
-                            out=out[b::bs], return_lse=False)
+                            out=out[b::bs], return_lse=False, q_prescaled=q_prescaled)
         return out
 
     def cross_attention(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor,
@@ -433,8 +440,8 @@ class FullyParallelAttention(torch.nn.Module):
             q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw)
             core = self._core_attention_fp8(q, kv, inference_params, meta_args, use_cache, core_dst)
         elif not use_cache:
-            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw)
-            core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst)
+            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw, q_premul=self._q_premul)
+            core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst, q_prescaled=True)
         else:
             if bs != 1 or inference_params.max_batch_size != 1:
                 raise ValueError("the cached path runs at batch 1 (as the reference pipeline does)")
@@ -451,16 +458,16 @@ class FullyParallelAttention(torch.nn.Module):
             if n_keep < S:
                 tail = torch.empty(S - n_keep, cache.shape[1], cache.shape[2], dtype=cache.dtype, device=cache.device)
             q, _ = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, kv_out=cache[start:], n_cache_rows=n_keep,
-                                   kv_tail=tail, raw=raw)
+                                   kv_tail=tail, raw=raw, q_premul=self._q_premul)
             split = start + n_keep
             kc, vc = cache[:split, :, :D], cache[:split, :, D:]
             if tail is None:
                 core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                          out=core_dst, return_lse=False)
+                                          out=core_dst, return_lse=False, q_prescaled=True)
             else:
                 core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
                                           k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, out=core_dst,
-                                          return_lse=False)
+                                          return_lse=False, q_prescaled=True)
         if fused is not None:
             self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, get_xqkv, out=cross_dst)
             return fused

@@ -135,8 +135,11 @@ def apply_rope_neox_partial(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tenso
 # --------------------------------------------------------------------------------------
 def prologue(q_raw: torch.Tensor, k_raw: torch.Tensor, v_raw: torch.Tensor, rope: torch.Tensor,
              gq: torch.Tensor, bq: torch.Tensor, gk: torch.Tensor, bk: torch.Tensor,
-             eps: float = 1e-6, norm: str = "layernorm_1p") -> Tuple[torch.Tensor, torch.Tensor]:
+             eps: float = 1e-6, norm: str = "layernorm_1p", q_premul: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
     """q_raw [S, Hq, D], k_raw / v_raw [S, Hkv, D] in bf16 (the projections' outputs, batch 1).
+
+    q_premul (no counterpart in the reference; 1.0 reproduces it): factor applied to q in fp32 ahead of the
+    downcast, for kernels that want softmax_scale * log2(e) folded into q.
 
     Returns (q [S, Hq, D] bf16, kv [S, Hkv, 2D] bf16) as get_q (:953-963) and get_kv (:991-996)
     do: upcast to fp32, norm, rotary in fp32, downcast to the input dtype; V is only
@@ -144,7 +147,7 @@ def prologue(q_raw: torch.Tensor, k_raw: torch.Tensor, v_raw: torch.Tensor, rope
     """
     sin, cos = rope.tensor_split(2, -1)
 
-    def one(x, g, b):
+    def one(x, g, b, premul=1.0):
         xf = x.float()
         if norm == "layernorm_1p":
             xf = qk_layernorm(xf, g.float(), b.float(), eps, True)
@@ -153,9 +156,11 @@ def prologue(q_raw: torch.Tensor, k_raw: torch.Tensor, v_raw: torch.Tensor, rope
         else:
             raise ValueError(norm)
         xf = apply_rope_neox_partial(xf, cos.float(), sin.float())
+        if premul != 1.0:
+            xf = xf * premul
         return xf.to(x.dtype)
 
-    q = one(q_raw, gq, bq)
+    q = one(q_raw, gq, bq, q_premul)
     k = one(k_raw, gk, bk)
     return q, torch.cat([k, v_raw], dim=-1)
 

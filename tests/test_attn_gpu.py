@@ -509,3 +509,31 @@ def test_every_workgroup_shape_on_the_small_cases(dev, monkeypatch, block_m):
     out2, _ = M.range_attention(q.to(dev), cache[:split, :, :128], cache[:split, :, 128:], tq, tk, L,
                                 k2=cache[split:, :, :128], v2=cache[split:, :, 128:], k_split=split, return_lse=False)
     _cmp(out2, ref, f"block_m={block_m} two segments")
+
+
+@pytest.mark.parametrize("block_m", ["384", "128"])
+def test_prescaled_q_flag(dev, monkeypatch, block_m):
+    """q_prescaled: q carries softmax_scale * log2(e), so q . k is the exp2 exponent.  The 12-wave kernel has an
+    instantiation that then accumulates the score MFMAs onto the negated running maximum; every other one runs with
+    a unit score scale.  Oracle on the same pre-scaled bf16 q with softmax_scale = ln 2 (2^x = e^(x ln 2)); lse
+    likewise.  Includes large scores (no multiply in fp32 is there to absorb them) and a first tile far below 0."""
+    import math
+
+    monkeypatch.setenv("MAGI_ATTN_BLOCK_M", block_m)
+    cs = 128 ** -0.5 * math.log2(math.e)
+    for L, dn, sp, Hq, Hkv, gain in [(200, 3, 1, 6, 2, 1.0), (77, 2, 2, 3, 1, 1.0), (1536, 3, 0, 24, 8, 1.0),
+                                     (300, 2, 1, 4, 4, 12.0), (130, 1, 0, 2, 1, -9.0)]:
+        q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=515 + L)
+        if gain < 0:  # q anti-parallel to every key: all exponents far below the initial maximum 0
+            k = (k.float().abs() * 0 + k.float()[:1, :1].sign() * 2).bfloat16().expand_as(k).contiguous()
+            q = (-k[:1, :1].float() * abs(gain)).bfloat16().expand(dn * L, Hq, 128).contiguous()
+            v = torch.randn(v.shape, generator=torch.Generator().manual_seed(5)).bfloat16()
+        qp = (q.float() * (cs * (gain if gain > 0 else 1.0))).bfloat16()
+        qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+        tq, tk = _ranges(dev, qr, kr)
+        out, lse = M.range_attention(qp.to(dev), k.to(dev), v.to(dev), tq, tk, L, q_prescaled=True, softmax_scale=123.0)
+        ref = O.range_attention(qp, k, v, qr, kr, softmax_scale=math.log(2.0))
+        assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+        _cmp(out, ref, f"block_m={block_m} L={L} gain={gain}")
+        lse_ref = O.range_attention_lse(qp, k, v, qr, kr, softmax_scale=math.log(2.0))
+        assert (lse.cpu() - lse_ref).abs().max() < 5e-3 * max(1.0, lse_ref.abs().max().item() / 50)

@@ -54,6 +54,33 @@ def test_prologue_parity(dev, T, H, W, sp, dn, Hq, Hkv):
     assert torch.equal(kv[..., D:].cpu(), kv_ref[..., D:])  # V is a copy: bit exact
 
 
+def test_prologue_folds_a_factor_into_q_ahead_of_the_rounding(dev):
+    """q_premul (softmax_scale * log2(e) for the pre-scaled attention path): applied in fp32 after norm and rotary,
+    so q is rounded to bf16 once; K and V are untouched.  End to end: prologue with the factor + attention with
+    q_prescaled against the oracle's unscaled prologue + attention."""
+    import math
+
+    T, H, W, sp, dn, Hq, Hkv = 4, 5, 6, 1, 2, 6, 2
+    S, D = T * H * W, 128
+    L = S // dn
+    cs = D ** -0.5 * math.log2(math.e)
+    qr, kr, vr, (gq, bq, gk, bk) = _inputs(S, Hq, Hkv, seed=99)
+    rope = O.rope_for_forward(T, H, W, sp, dn)
+    shaped = (qr.view(S, Hq, D), kr.view(S, Hkv, D), vr.view(S, Hkv, D), rope, gq, bq, gk, bk)
+    q_ref, kv_ref = O.prologue(*shaped, q_premul=cs)
+    q_plain, _ = O.prologue(*shaped)
+    to = lambda t: t.to(dev)
+    q, kv, _ = M.qk_prologue(to(qr), to(kr), to(vr), to(rope), to(gq), to(bq), to(gk), to(bk), Hq=Hq, Hkv=Hkv, q_premul=cs)
+    _ulp_check(q, q_ref, "q * premul")
+    _ulp_check(kv[..., :D], kv_ref[..., :D], "k")
+    assert torch.equal(kv[..., D:].cpu(), kv_ref[..., D:])
+    ranges = [[0, L], [L, S]], [[0, L], [0, S]]
+    tq, tk = (torch.tensor(r, dtype=torch.int32, device=dev) for r in ranges)
+    out, _ = M.range_attention(q, kv[..., :D], kv[..., D:], tq, tk, L, q_prescaled=True, return_lse=False)
+    ref = O.range_attention(q_plain, kv_ref[..., :D], kv_ref[..., D:], *ranges)
+    assert (out.float().cpu() - ref).abs().max() <= 2e-2
+
+
 def test_prologue_rmsnorm_no_rope_and_strided_inputs(dev):
     S, Hq, Hkv, D = 50, 6, 2, 128
     qr, kr, vr, (gq, bq, gk, bk) = _inputs(S, Hq, Hkv, seed=3)

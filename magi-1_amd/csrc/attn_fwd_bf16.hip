@@ -28,7 +28,9 @@
 //     four statically named slots, one barrier per tile): every K / V tile is fetched from L2 once
 //     for 384 query rows instead of 128.  On grids of many rounds with long key ranges this is the
 //     faster one, although it needs more cycles: the part is power limited, and the bytes it does
-//     not move come back as clock.
+//     not move come back as clock.  Its PRESC form takes q already multiplied by softmax_scale *
+//     log2(e) (the prologue does that ahead of q's rounding to bf16) and accumulates the score
+//     MFMAs onto the negated running maximum, so the MFMA result is the exp2 argument.
 // Instantiations with 2 waves / SIMD (deep prefetch, K and V double buffered), with 32-key tiles,
 // with 8-wave workgroups, and a software-pipelined loop (PIPE: score MFMAs of the next tile, softmax
 // and PV MFMAs of the current one interleaved in one basic block, 2 waves / SIMD) are kept for

@@ -227,6 +227,20 @@ def _full_size_check(dev, L, dn, sp, Hq, Hkv, seed, rows_per_chunk, cpu_rows):
     ones[..., D:] = 1
     o1, _ = M.range_attention(q, ones[..., :D], ones[..., D:], tq, tk, L, return_lse=False)
     assert (o1.float() - 1).abs().max() <= 2 ** -7
+    del ones, o1
+    # the pre-scaled path (q carries softmax_scale * log2(e)) at the same size, on the last chunk's subsample
+    import math
+    qp = (q.float() * (D ** -0.5 * math.log2(math.e))).bfloat16()
+    outp, _ = M.range_attention(qp, cache[..., :D], cache[..., D:], tq, tk, L, q_prescaled=True, return_lse=False)
+    i = dn - 1
+    rows = torch.tensor(np.sort(rs.choice(L, rows_per_chunk, replace=False)) + i * L, device=dev)
+    ke = int(kr[i, 1])
+    ref = torch.empty(rows_per_chunk, Hq, D, device=dev)
+    for hk in range(Hkv):
+        kk, vv = cache[:ke, hk, :D].float(), cache[:ke, hk, D:].float()
+        s2 = torch.einsum("rgd,kd->rgk", qp[rows][:, hk * G:(hk + 1) * G].float(), kk) * math.log(2.0)
+        ref[:, hk * G:(hk + 1) * G] = torch.einsum("rgk,kd->rgd", torch.softmax(s2, -1), vv)
+    _cmp(outp[rows], ref, "pre-scaled q, GPU fp32 subsample")
 
 
 def test_full_size_480p_layer(dev):

@@ -23,14 +23,15 @@
 // shallow operand prefetch):
 //   * 4 waves per workgroup, three workgroups per CU, 48 KB of LDS each (64-key tiles, K double
 //     buffered, ONE V slot that is refilled under the score MFMAs and the softmax of the same tile,
-//     two barriers per tile): small grids and short key ranges;
+//     two barriers per tile, slots named statically): small grids and short key ranges;
 //   * 12 waves per workgroup (DB), ONE workgroup per CU, 64 KB of LDS (K and V double buffered in
 //     four statically named slots, one barrier per tile): every K / V tile is fetched from L2 once
 //     for 384 query rows instead of 128.  On grids of many rounds with long key ranges this is the
 //     faster one, although it needs more cycles: the part is power limited, and the bytes it does
-//     not move come back as clock.  Its PRESC form takes q already multiplied by softmax_scale *
-//     log2(e) (the prologue does that ahead of q's rounding to bf16) and accumulates the score
-//     MFMAs onto the negated running maximum, so the MFMA result is the exp2 argument.
+//     not move come back as clock.
+// Both have a PRESC form that takes q already multiplied by softmax_scale * log2(e) (the prologue
+// does that ahead of q's rounding to bf16) and accumulates the score MFMAs onto the negated running
+// maximum, so the MFMA result is the exp2 argument and no per-score multiply-subtract remains.
 // Instantiations with 2 waves / SIMD (deep prefetch, K and V double buffered), with 32-key tiles,
 // with 8-wave workgroups, and a software-pipelined loop (PIPE: score MFMAs of the next tile, softmax
 // and PV MFMAs of the current one interleaved in one basic block, 2 waves / SIMD) are kept for
@@ -121,9 +122,9 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");
   static_assert(!PIPE || (NSTAGE == 2 && BN == 64 && !VSINGLE), "pipelined loop: 64-key tiles, two K slots and two V slots");
   static_assert(!DB || (NSTAGE == 2 && !VSINGLE && !PIPE), "static double buffer: two K slots and two V slots");
-  // ring of NSTAGE (K tile, V tile) pairs, or in single-V mode K slot 0, K slot 1, V slot
-  // (the pipelined loop declares its four slots as separate objects instead and leaves this one a stub)
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[(PIPE || DB) ? 1 : VSINGLE ? 3 : 2 * NSTAGE][(PIPE || DB) ? 16 : TILE_BYTES];
+  // ring of NSTAGE (K tile, V tile) pairs for the loops that index their slots at run time; the single-V, the
+  // double-buffered and the pipelined loops declare their slots as separate objects and leave this one a stub
+  __shared__ __attribute__((aligned(1024))) unsigned char smem[(PIPE || DB || VSINGLE) ? 1 : 2 * NSTAGE][(PIPE || DB || VSINGLE) ? 16 : TILE_BYTES];
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -624,26 +625,43 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       if (it + 1 >= n_tiles) break;
       step(it + 1, std::integral_constant<int, 1>{});
     }
+  } else if constexpr (VSINGLE) {
+    // single-V mode (48 KB of LDS, three workgroups per CU) with statically named slots, the loop unrolled by two:
+    // K(it) was requested one iteration ago; V(it) is requested now, into the one V slot that PV(it-1) has just
+    // released, and lands under the score MFMAs and the softmax of this tile; a second barrier publishes it
+    // before PV(it).
+    __shared__ __attribute__((aligned(1024))) unsigned char vK0[TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char vK1[TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) unsigned char vV[TILE_BYTES];
+    issue_mat(ks, vK0, false);
+    auto step = [&](int it, auto bc) {
+      constexpr int B = decltype(bc)::value;
+      const int k0 = ks + it * BN;
+      wait_vmcnt<0>();
+      __syncthreads();
+      issue_mat(k0, vV, true);
+      if (it + 1 < n_tiles) issue_mat(k0 + BN, B ? vK0 : vK1, false);
+      compute_tile(B ? vK1 : vK0, vV, k0, [&]() {
+        if (it + 1 < n_tiles)
+          wait_vmcnt<LOADS>();  // V(it) landed; the K(it+1) loads issued after it may still be in flight
+        else
+          wait_vmcnt<0>();
+        __syncthreads();
+      });
+    };
+    for (int it = 0; it < n_tiles; it += 2) {
+      step(it, std::integral_constant<int, 0>{});
+      if (it + 1 >= n_tiles) break;
+      step(it + 1, std::integral_constant<int, 1>{});
+    }
   } else {
-  if (VSINGLE) {
-    issue_mat(ks, &smem[0][0], false);
-  } else {
+    // ring of NSTAGE (K tile, V tile) pairs, tiles requested NSTAGE-1 ahead, one barrier per tile
 #pragma unroll
     for (int p = 0; p < NSTAGE - 1; ++p)
       if (p < n_tiles) issue_tile(ks + p * BN, p);
-  }
-  int stage = 0;
-  for (int it = 0; it < n_tiles; ++it) {
-    const int k0 = ks + it * BN;
-    if (VSINGLE) {
-      // single-V mode (48 KB of LDS, three workgroups per CU): K(it) was requested one iteration ago; V(it)
-      // is requested now, into the one V slot that PV(it-1) has just released, and lands under the score
-      // MFMAs and the softmax of this tile; a second barrier publishes it before PV(it).
-      wait_vmcnt<0>();
-      __syncthreads();
-      issue_mat(k0, &smem[2][0], true);
-      if (it + 1 < n_tiles) issue_mat(k0 + BN, &smem[(it + 1) & 1][0], false);
-    } else {
+    int stage = 0;
+    for (int it = 0; it < n_tiles; ++it) {
+      const int k0 = ks + it * BN;
       // tile `it` must have landed; up to NSTAGE-2 younger tiles may still be in flight
       const int younger = min(NSTAGE - 2, n_tiles - 1 - it);
       if (NSTAGE >= 4 && younger == 2)
@@ -658,22 +676,12 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
         if (st >= NSTAGE) st -= NSTAGE;
         issue_tile(k0 + (NSTAGE - 1) * BN, st);
       }
+      const unsigned char* Kt = &smem[2 * stage][0];
+      const unsigned char* Vt = &smem[2 * stage + 1][0];
+      stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
+      if (!wave_on) continue;
+      compute_tile(Kt, Vt, k0, []() {});
     }
-    const unsigned char* Kt = &smem[VSINGLE ? (it & 1) : 2 * stage][0];
-    const unsigned char* Vt = &smem[VSINGLE ? 2 : 2 * stage + 1][0];
-    stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
-    if (!VSINGLE && !wave_on) continue;
-
-    compute_tile(Kt, Vt, k0, [&]() {
-      if (VSINGLE) {
-        if (it + 1 < n_tiles)
-          wait_vmcnt<LOADS>();  // V(it) landed; the K(it+1) loads issued after it may still be in flight
-        else
-          wait_vmcnt<0>();
-        __syncthreads();
-      }
-    });
-  }
   }  // !DB
   }  // !PIPE
 
@@ -716,6 +724,8 @@ hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false>), dim3(grid), dim3(256), 0, stream, a);
   else if (a.variant == 3)  // software-pipelined loop, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false, true>), dim3(grid), dim3(256), 0, stream, a);
+  else if ((a.flags & 2) && a.variant != 7)  // 4 waves, q pre-scaled (PRESC)
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true, false, false, true>), dim3(grid), dim3(256), 0, stream, a);
   else  // 4 waves, 64-key tiles, double-buffered K, single V slot, three workgroups per CU
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();

@@ -26,6 +26,9 @@ Pin status (what besides "same formula" checks each function; see tests/test_ora
   kv-range generators               hand-derived expected tables
   fp8 quantiser / fp8 attention     PARITY UNPINNED by the reference (it has no fp8 attention);
                                     pinned by quantiser properties and the fp32 oracle + tolerance
+  prologue(q_premul != 1)           no counterpart in the reference (1.0 reproduces it); pinned end to end: the
+                                    pre-scaled q through attention with softmax_scale = ln 2 must equal the
+                                    unscaled prologue + default-scale attention (tests/test_oracle.py)
 """
 from __future__ import annotations
 

@@ -379,3 +379,31 @@ def test_fp8_quantiser_properties():
     rel = (back - t).abs() / t.abs().clamp_min(1e-3 * t.abs().amax())
     assert (back - t).abs().max() <= 0.0625 * t.abs().max() + 1e-6  # e4m3: 3 mantissa bits
     assert t8.float().abs().max() == 448  # absmax maps onto the top code
+
+
+def test_prologue_premul_is_the_softmax_scale_moved_into_q():
+    """prologue(q_premul=c) has no counterpart in the reference.  Pin: with c = softmax_scale * log2(e) the
+    pre-scaled q through attention with softmax_scale = ln 2 equals (up to q's bf16 rounding) the reference-shaped
+    unscaled prologue followed by default-scale attention; K, V are untouched; c = 1 is the plain prologue; and in
+    fp32 (no rounding) the factor commutes exactly: prologue(x, c) == c * prologue(x)."""
+    g = torch.Generator().manual_seed(3)
+    T, H, W, Hq, Hkv, D = 2, 3, 4, 4, 2, 128
+    S = T * H * W
+    rope = O.rope_for_forward(T, H, W, 0, 1)
+    mk = lambda *s: torch.randn(*s, generator=g)
+    gq, bq, gk, bk = (mk(D) * 0.1 for _ in range(4))
+    q_raw, k_raw, v_raw = mk(S, Hq, D).bfloat16(), mk(S, Hkv, D).bfloat16(), mk(S, Hkv, D).bfloat16()
+    c = D ** -0.5 * math.log2(math.e)
+    q0, kv0 = O.prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk)
+    q1, kv1 = O.prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, q_premul=c)
+    qa, kva = O.prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, q_premul=1.0)
+    assert torch.equal(kv0, kv1) and torch.equal(q0, qa) and torch.equal(kv0, kva)
+    qf0, _ = O.prologue(q_raw.float(), k_raw.float(), v_raw.float(), rope, gq, bq, gk, bk)
+    qf1, _ = O.prologue(q_raw.float(), k_raw.float(), v_raw.float(), rope, gq, bq, gk, bk, q_premul=c)
+    assert torch.allclose(qf1, qf0 * c, rtol=1e-6, atol=0)
+    # one rounding to bf16 on each side: half an ulp (2^-8 relative) each
+    assert (q1.float() - q0.float() * c).abs().max() <= 2 * 2 ** -8 * (q0.float().abs().max() * c)
+    r = [[0, S]]
+    a = O.range_attention(q0, kv0[..., :D], kv0[..., D:], r, r)
+    b = O.range_attention(q1, kv1[..., :D], kv1[..., D:], r, r, softmax_scale=math.log(2.0))
+    assert (a - b).abs().max() < 5e-3

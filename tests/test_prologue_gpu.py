@@ -402,6 +402,10 @@ def test_layer_with_fp8_self_attention_and_fp8_cache(dev):
             core, xo = fp8_layer(hs, y, ip_fp8 if has_ip else None, rope, meta)
             vmax = ref_layer.linear_qkv.forward_v(ref_layer.linear_qkv.forward_ln(hs)).float().abs().max().item()
         assert torch.equal(xo, xo_ref)
+        if not has_ip:  # (a pass that leaves the caches alone) the fp8 path writes the linear_proj layout too
+            with torch.no_grad():
+                fused = fp8_layer(hs, y, None, rope, meta, proj_layout=True)
+            assert torch.equal(fused, MOD.attn_linear_proj_input(core, xo))
         a, b = core.double().flatten(), core_ref.double().flatten()
         cos = (a @ b / (a.norm() * b.norm())).item()
         err = (a - b).abs().max().item()

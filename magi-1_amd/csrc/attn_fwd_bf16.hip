@@ -115,8 +115,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   constexpr int TILE_LOADS = 2 * LOADS;    // ... per wave per tile
   constexpr int NT = BN / 32;              // 32-key score tiles per key tile
   constexpr int NS = BN / 16;              // 16-key slabs per key tile
-  constexpr int DK = PRESC ? 2 : WPS >= 3 ? 4 : 8;  // K operands in flight
-  constexpr int DV = PRESC ? 2 : WPS >= 3 ? 4 : 8;  // V operands in flight
+  constexpr int DK = WPS >= 3 ? 4 : 8;     // K operands in flight
+  constexpr int DV = WPS >= 3 ? 4 : 8;     // V operands in flight
   constexpr bool VEARLY = !VSINGLE && WPS < 3;  // first V operands fetched under the last score MFMAs (needs registers)
   static_assert(LOADS >= 1 && NSTAGE >= 2 && NSTAGE <= 4, "bad tile configuration");
   static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");

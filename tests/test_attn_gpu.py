@@ -2,6 +2,7 @@
 
 Tolerance (bf16 path, from the benchmark definition): max-abs <= 2e-2 and cosine >= 0.9999
 against the fp32 reference on identical seeded inputs."""
+import math
 import os
 
 import numpy as np
@@ -370,7 +371,10 @@ def test_randomised_shapes_ranges_strides_and_splits(dev):
         ks = rng.integers(0, Tk, size=n)
         kr = np.stack([ks, np.minimum(Tk, ks + rng.integers(0, 400, size=n))], 1)
         q, k, v = O.synthetic_qkv(Tq, Tk, Hq, Hkv, 128, seed=5000 + case)
-        ref = O.range_attention(q, k, v, qr, kr)
+        prescaled = case % 5 in (1, 3)  # q carries softmax_scale * log2(e): the oracle then runs with scale ln 2
+        if prescaled:
+            q = (q.float() * (128 ** -0.5 * math.log2(math.e))).bfloat16()
+        ref = O.range_attention(q, k, v, qr, kr, softmax_scale=math.log(2.0) if prescaled else None)
         covered = np.zeros(Tq, bool)
         for a, b in qr:
             covered[a:b] = True
@@ -392,7 +396,7 @@ def test_randomised_shapes_ranges_strides_and_splits(dev):
             split = int(rng.integers(0, Tk + 1))
             kw = dict(k2=kd[split:], v2=vd[split:], k_split=split)  # same strides as the first segment
             kd, vd = kd[:split], vd[:split]
-        out, lse = M.range_attention(q.to(dev), kd, vd, tq, tk, int(ql.max()), **kw)
+        out, lse = M.range_attention(q.to(dev), kd, vd, tq, tk, int(ql.max()), q_prescaled=prescaled, **kw)
         cov = torch.tensor(covered, device=dev)
         if torch.count_nonzero(ref).item() == 0:  # every range of this case is empty
             assert torch.count_nonzero(out).item() == 0

@@ -192,6 +192,30 @@ def cpu_baseline(inp, rows_per_chunk=6144):
                        f"{fl:.3e} FLOP in {dt:.1f} s (torch {torch.__version__} CPU SDPA fp32)"), o, idx
 
 
+def layer_norm_leg(inp, steps):
+    """The LayerNorm of the layer input (the step ahead of the projections that feed the prologue), kernel-only:
+    reported beside the headline, not part of `value`.  Re-uses the raw-q buffer as the hidden states and the
+    cross-attention output buffer for the result (nothing reads that buffer afterwards)."""
+    import magi_attn as M
+
+    S, hidden = inp["S"], inp["Hq"] * inp["D"]
+    x, y = inp["q_raw"], inp["xout"].view(S, hidden)
+    w = torch.ones(hidden, dtype=torch.bfloat16, device=x.device)
+    b = torch.zeros(hidden, dtype=torch.bfloat16, device=x.device)
+    for _ in range(2):
+        M.layer_norm(x, w, b, 1e-6, out=y)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        M.layer_norm(x, w, b, 1e-6, out=y)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / steps
+    gbs = 2 * S * hidden * 2 / (ms * 1e-3) / 1e9
+    return {"bound": "hbm", "kernel": "layer_norm_kernel", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
+            "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "ms": round(ms, 4)}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -264,6 +288,7 @@ def main():
     }
     if not args.no_fp8:
         result["fp8"] = fp8_leg(inp, core_fl, core_tflops, args.steps)
+    result["roofline_layer_norm"] = layer_norm_leg(inp, args.steps)
     if args.copy_calibration:
         inp["xout"].copy_(inp["out"])  # reads and writes out.numel() * 2 bytes each
         torch.cuda.synchronize()

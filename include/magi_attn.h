@@ -166,6 +166,17 @@ typedef struct magi_prologue_args {
 int magi_qk_prologue(const magi_prologue_args* args, void* stream);
 
 /*
+ * LayerNorm of the layer input over its last axis: x [rows, cols] bf16 -> y [rows, cols] bf16 with fp32
+ * statistics, y = (x - mean) / sqrt(var + eps) * weight + bias (plain weight, not the "+1" form).
+ * Stands in for torch.nn.LayerNorm in CustomLayerNormLinear.forward_ln (dit_module.py:401, 412-413;
+ * first step of the layer forward, :1153).  weight / bias [cols] are bf16 (params_fp32 == 0, the
+ * reference's params_dtype) or fp32; NULL weight = 1, NULL bias = 0.  Row strides in elements.
+ * cols: multiples of 8 up to 8192.
+ */
+int magi_layer_norm(const void* x, int64_t x_stride, const void* weight, const void* bias, int32_t params_fp32,
+                    void* y, int64_t y_stride, int64_t rows, int32_t cols, float eps, void* stream);
+
+/*
  * Per-head norm only (no rotary, no cache): x [S, H, D] bf16 -> y [S, H, D] bf16, computed in the
  * precision the reference uses for the cross-attention norms (bf16 in, fp32 statistics, bf16 out).
  * Stands in for q_layernorm_xattn / k_layernorm_xattn in get_xqkv (dit_module.py:1008, 1020).

@@ -214,6 +214,24 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   return MAGI_OK;
 }
 
+int magi_layer_norm(const void* x, int64_t x_stride, const void* weight, const void* bias, int32_t params_fp32,
+                    void* y, int64_t y_stride, int64_t rows, int32_t cols, float eps, void* stream) {
+  if (rows < 0 || cols < 0) return fail(MAGI_EINVAL, "magi_layer_norm: negative size");
+  if (rows == 0 || cols == 0) return MAGI_OK;
+  if (cols % 8 || cols > 8192)
+    return fail(MAGI_ENOSYS, "magi_layer_norm: cols %d not implemented (multiples of 8 up to 8192)", cols);
+  if (!x || !y) return fail(MAGI_EINVAL, "magi_layer_norm: NULL x/y");
+  if (x_stride < cols || y_stride < cols) return fail(MAGI_EINVAL, "magi_layer_norm: row stride below cols");
+  if (x_stride % 8 || y_stride % 8 || !aligned16(x) || !aligned16(y))
+    return fail(MAGI_EINVAL, "magi_layer_norm: rows must be 16-byte aligned");
+  if (!(eps >= 0.f)) return fail(MAGI_EINVAL, "magi_layer_norm: eps");
+  hipError_t e = magi::launch_layer_norm(static_cast<const char*>(x), x_stride * 2, weight, bias, params_fp32 != 0,
+                                         static_cast<char*>(y), y_stride * 2, rows, cols, eps, compute_units(),
+                                         static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "magi_layer_norm launch");
+  return MAGI_OK;
+}
+
 int magi_head_norm(const void* x, int64_t x_stride_t, int64_t x_stride_h, const float* gamma, const float* beta,
                    void* y, int32_t S, int32_t H, int32_t D, int32_t norm_kind, float eps, void* stream) {
   if (D != 128) return fail(MAGI_ENOSYS, "magi_head_norm: head_dim %d not implemented (128 only)", D);

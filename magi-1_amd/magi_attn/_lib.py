@@ -61,7 +61,7 @@ class PrologueArgs(C.Structure):
 
 
 EXPORTS = ("magi_version", "magi_last_error", "magi_attn_fwd", "magi_qk_prologue", "magi_head_norm",
-           "magi_apply_rotary", "magi_quantize_fp8")
+           "magi_apply_rotary", "magi_quantize_fp8", "magi_layer_norm")
 
 _lib = None
 
@@ -84,6 +84,9 @@ def lib() -> C.CDLL:
         l.magi_head_norm.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,
                                      C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_void_p]
         l.magi_head_norm.restype = C.c_int
+        l.magi_layer_norm.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int64,
+                                      C.c_int64, C.c_int32, C.c_float, C.c_void_p]
+        l.magi_layer_norm.restype = C.c_int
         l.magi_apply_rotary.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                         C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
         l.magi_apply_rotary.restype = C.c_int

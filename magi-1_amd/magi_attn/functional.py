@@ -252,6 +252,40 @@ def qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int,
     return q_out, kv_out, kv_tail
 
 
+def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float = 1e-5,
+               out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """LayerNorm over the last axis of a bf16 tensor with fp32 statistics: the layer input norm of
+    CustomLayerNormLinear.forward_ln (dit_module.py:401, 412-413).  weight / bias: bf16 or fp32 [cols] or None.
+    Rows may be strided (last axis contiguous, leading axes collapsible to one row stride)."""
+    if x.dtype != torch.bfloat16:
+        raise TypeError("x must be bf16")
+    if not x.is_cuda:
+        raise ValueError("x must be a device tensor (there is no CPU path)")
+    cols = x.shape[-1]
+    x2 = x if x.dim() == 2 else x.reshape(-1, cols)  # a view when the leading axes collapse, else a copy
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    y = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device) if out is None else out
+    if y.shape != x.shape or y.dtype != torch.bfloat16 or y.device != x.device or not y.is_contiguous():
+        raise ValueError("out must be a contiguous bf16 tensor of x's shape on x's device")
+    fp32 = None
+    for name, p in (("weight", weight), ("bias", bias)):
+        if p is None:
+            continue
+        if p.shape != (cols,) or not p.is_contiguous() or p.device != x.device:
+            raise ValueError(f"{name} must be a contiguous [{cols}] tensor on x's device")
+        if p.dtype not in (torch.bfloat16, torch.float32):
+            raise TypeError(f"{name} must be bf16 or fp32")
+        if fp32 is not None and fp32 != (p.dtype == torch.float32):
+            raise TypeError("weight and bias must share a dtype")
+        fp32 = p.dtype == torch.float32
+    rows = x2.shape[0]
+    with torch.cuda.device(x.device):
+        L.check(L.lib().magi_layer_norm(x2.data_ptr(), x2.stride(0) if rows > 1 else cols, _ptr(weight), _ptr(bias),
+                                        int(bool(fp32)), y.data_ptr(), cols, rows, cols, float(eps), _stream()))
+    return y
+
+
 def head_norm(x: torch.Tensor, gamma, beta, eps: float = 1e-6, norm_kind: int = L.MAGI_NORM_LAYERNORM_1P):
     """x [S, H, 128] bf16 (strided heads allowed) -> contiguous normalised copy."""
     _check_thd(x, "x")

@@ -32,7 +32,7 @@ import math
 
 from . import _lib as L
 from .cache import Fp8KVCache
-from .functional import head_norm, qk_prologue, quantize_fp8, range_attention
+from .functional import head_norm, layer_norm, qk_prologue, quantize_fp8, range_attention
 from .params import InferenceParams, ModelMetaArgs, PackedCrossAttnParams
 
 
@@ -130,7 +130,10 @@ class CustomLayerNormLinear(torch.nn.Module):
         return y[..., :oq], y[..., oq:oq + okv], y[..., oq + okv:oq + 2 * okv], y[..., oq + 2 * okv:]
 
     def forward_ln(self, hidden_states):
-        return self.layer_norm(hidden_states)
+        """LayerNorm of the layer input (dit_module.py:412-413) as one HIP launch; the parameters stay on the
+        torch.nn.LayerNorm sub-module under the reference's names."""
+        ln = self.layer_norm
+        return layer_norm(hidden_states, ln.weight.detach(), ln.bias.detach(), ln.eps)
 
     def forward_q(self, hidden_states):
         return self.q(hidden_states)

@@ -16,6 +16,7 @@ Pin status (what besides "same formula" checks each function; see tests/test_ora
   freq_bands, rope_table            closed-form spot values, axis-separability, symmetry,
                                     identity rescale for H*W == 256, slice == offset-table
   qk_layernorm / rmsnorm            torch.nn.functional.layer_norm with weight+1; fp64 brute force
+  input_layer_norm                  torch.nn.LayerNorm module (CPU, fp32), shift / scale invariances
   apply_rope_neox_partial           transformers' rotate_half convention, pair-norm invariance,
                                     pass-through dims, relative-position property
   range_attention                   fp64 brute force, block-mask SDPA, V=1 => O=1, permutation
@@ -109,6 +110,22 @@ def qk_layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps:
     """LayerNorm over the last (head_dim) axis with gamma stored zero-centred (:356-357)."""
     w = weight + 1 if zero_centered_gamma else weight
     return F.layer_norm(x, (x.shape[-1],), w, bias, eps)
+
+
+def input_layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+                     eps: float = 1e-5) -> torch.Tensor:
+    """LayerNorm of the layer input over the hidden axis (torch.nn.LayerNorm in CustomLayerNormLinear,
+    dit_module.py:401, applied at :412-413 / :1153): biased variance, plain (not zero-centred) weight.
+    Evaluated in float64 from the definition; the caller rounds to the dtype under test."""
+    xd = x.double()
+    mu = xd.mean(-1, keepdim=True)
+    var = ((xd - mu) ** 2).mean(-1, keepdim=True)
+    y = (xd - mu) / torch.sqrt(var + eps)
+    if weight is not None:
+        y = y * weight.double()
+    if bias is not None:
+        y = y + bias.double()
+    return y
 
 
 def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor] = None, eps: float = 1e-6) -> torch.Tensor:

@@ -95,6 +95,16 @@ def test_prologue_argument_validation_without_gpu():
     p.R2 = 48
     assert lib.magi_qk_prologue(C.byref(p), None) == -22  # NULL buffers
     assert lib.magi_head_norm(None, 0, 0, None, None, None, 4, 2, 128, 0, 1e-6, None) == -22
+    # layer norm: validation happens before any device work
+    buf = (C.c_char * 64)()
+    p16 = (C.addressof(buf) + 15) & ~15
+    assert lib.magi_layer_norm(None, 64, None, None, 0, None, 64, 0, 64, 1e-5, None) == 0  # no rows: nothing to do
+    assert lib.magi_layer_norm(None, 64, None, None, 0, None, 64, 4, 64, 1e-5, None) == -22
+    assert lib.magi_layer_norm(p16, 64, None, None, 0, p16, 64, 4, 60, 1e-5, None) == -38  # cols % 8
+    assert lib.magi_layer_norm(p16, 64, None, None, 0, p16, 64, 4, 8200, 1e-5, None) == -38
+    assert lib.magi_layer_norm(p16, 32, None, None, 0, p16, 64, 4, 64, 1e-5, None) == -22  # stride < cols
+    assert lib.magi_layer_norm(p16 + 2, 64, None, None, 0, p16, 64, 4, 64, 1e-5, None) == -22  # alignment
+    assert b"magi_layer_norm" in lib.magi_last_error()
     assert lib.magi_apply_rotary(None, None, None, None, 1, 4, 2, 128, 80, 0, None) == -22
 
 

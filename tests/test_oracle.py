@@ -98,6 +98,25 @@ def test_qk_layernorm_vs_fp64_definition():
     assert torch.allclose(y0.var(-1, unbiased=False), torch.ones(7, 3), atol=1e-4)
 
 
+def test_input_layer_norm_vs_torch_module_and_invariances():
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(9, 384, generator=g) * 3 + 0.7
+    ln = torch.nn.LayerNorm(384, eps=1e-5)
+    with torch.no_grad():
+        ln.weight.copy_(torch.randn(384, generator=g))
+        ln.bias.copy_(torch.randn(384, generator=g))
+        ref = ln(x)
+    y = O.input_layer_norm(x, ln.weight.detach(), ln.bias.detach(), 1e-5)
+    assert (y - ref.double()).abs().max() < 2e-5
+    # without affine parameters: zero mean, unit (biased) variance, invariant to a shift and a positive scale
+    y0 = O.input_layer_norm(x, None, None, 0.0)
+    assert y0.mean(-1).abs().max() < 1e-12 and (y0.var(-1, unbiased=False) - 1).abs().max() < 1e-12
+    assert (O.input_layer_norm(4.0 * x + 2.5, None, None, 0.0) - y0).abs().max() < 1e-5
+    # eps enters under the root: a constant row maps to the bias
+    c = torch.full((2, 384), 3.25)
+    assert torch.equal(O.input_layer_norm(c, ln.weight.detach(), ln.bias.detach(), 1e-5), ln.bias.detach().double().expand(2, -1))
+
+
 def test_rmsnorm_unit_rms():
     x = torch.randn(5, 2, 128, generator=torch.Generator().manual_seed(1))
     y = O.rmsnorm(x)

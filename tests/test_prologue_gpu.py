@@ -422,3 +422,61 @@ def test_layer_with_fp8_self_attention_and_fp8_cache(dev):
             for got, ref_half in ((cache.k[rows].float() * sc(cache.k_scale), want[..., :D]),
                                   (cache.v[rows].float() * sc(cache.v_scale), want[..., D:])):
                 assert ((got - ref_half).abs() <= ref_half.abs() * 2 ** -4 + 2 ** -9 * ref_half.abs().max()).all()
+
+
+# ----------------------------------------------------------------------------- layer input norm
+@pytest.mark.parametrize("rows,cols,params", [
+    (1000, 6144, "bf16"), (333, 3072, "bf16"), (77, 4096, "fp32"), (5, 8, "bf16"), (64, 8192, "bf16"),
+    (100, 1000, "fp32"), (1, 520, "bf16"), (4099, 1536, "none"), (9000, 6144, "bf16"),
+])
+def test_layer_norm_matches_oracle(rows, cols, params):
+    """Layer input LayerNorm (dit_module.py:401, 412-413): fp32 statistics, one rounding to bf16.  The oracle
+    evaluates the definition in float64; bar as for the prologue (one bf16 ulp, < 1 in 1000 elements differ)."""
+    g = torch.Generator().manual_seed(rows * 31 + cols)
+    x = (torch.randn(rows, cols, generator=g) * 2.0 + 0.5).bfloat16()
+    dt = {"bf16": torch.bfloat16, "fp32": torch.float32, "none": None}[params]
+    w = None if dt is None else (1 + 0.3 * torch.randn(cols, generator=g)).to(dt)
+    b = None if dt is None else (0.2 * torch.randn(cols, generator=g)).to(dt)
+    dev = lambda t: None if t is None else t.cuda()
+    y = M.layer_norm(x.cuda(), dev(w), dev(b), 1e-5)
+    torch.cuda.synchronize()
+    assert y.shape == x.shape and y.dtype == torch.bfloat16
+    ref = O.input_layer_norm(x, w, b, 1e-5).float().bfloat16()
+    _ulp_check(y, ref, f"layer_norm {rows}x{cols} {params}")
+
+
+def test_layer_norm_strided_rows_leading_axes_and_offset_mean():
+    g = torch.Generator().manual_seed(77)
+    # rows that are column slices of a wider buffer, as a view of a fused activation would be
+    wide = torch.randn(301, 2 * 3072, generator=g).bfloat16()
+    w = (1 + 0.1 * torch.randn(3072, generator=g)).bfloat16()
+    b = (0.1 * torch.randn(3072, generator=g)).bfloat16()
+    y = M.layer_norm(wide.cuda()[:, 3072:], w.cuda(), b.cuda(), 1e-6)
+    _ulp_check(y, O.input_layer_norm(wide[:, 3072:], w, b, 1e-6).float().bfloat16(), "strided rows")
+    # [sq, b, h] input as the layer passes it, written into a caller's buffer
+    x3 = torch.randn(50, 2, 1024, generator=g).bfloat16()
+    out = torch.empty(50, 2, 1024, dtype=torch.bfloat16, device="cuda")
+    y3 = M.layer_norm(x3.cuda(), w.cuda()[:1024].contiguous(), None, 1e-6, out=out)
+    assert y3 is out
+    _ulp_check(y3, O.input_layer_norm(x3, w[:1024], None, 1e-6).float().bfloat16(), "3-d input")
+    # a mean far above the spread: the two-pass variance must not cancel
+    xo = (torch.randn(40, 2048, generator=g) * 0.25 + 100.0).bfloat16()
+    yo = M.layer_norm(xo.cuda(), None, None, 1e-5)
+    _ulp_check(yo, O.input_layer_norm(xo, None, None, 1e-5).float().bfloat16(), "offset mean")
+    # a constant row: zero variance, the result is the bias
+    c = torch.full((3, 512), 1.5).bfloat16()
+    yc = M.layer_norm(c.cuda(), w.cuda()[:512].contiguous(), b.cuda()[:512].contiguous(), 1e-5)
+    assert torch.equal(yc.cpu(), b[:512].expand(3, -1))
+
+
+def test_layer_norm_rejects_bad_arguments():
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(TypeError):
+        M.layer_norm(x.float(), None, None)
+    with pytest.raises(ValueError):
+        M.layer_norm(x, torch.ones(32, dtype=torch.bfloat16, device="cuda"), None)
+    with pytest.raises(TypeError):
+        M.layer_norm(x, torch.ones(64, dtype=torch.bfloat16, device="cuda"), torch.ones(64, device="cuda"))
+    with pytest.raises(M.MagiError):
+        M.layer_norm(torch.zeros(4, 60, dtype=torch.bfloat16, device="cuda"), None, None)
+    assert M.layer_norm(x[:0], None, None).shape == (0, 64)

@@ -31,7 +31,8 @@ PEAK_HBM_GBS = 8000.0
 Q_PREMUL = 128 ** -0.5 * math.log2(math.e)  # softmax_scale * log2(e) at head_dim 128
 # HBM-side bytes per launch on the 720p workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # plain copy of known size in the same run (FETCH_SIZE x2.0, WRITE_SIZE x1.0): profiles/bench_720p_hbm_traffic_pmc.txt
-MEASURED_TRAFFIC = {"720p-24B": {"core": 186.8e9 + 1.07e9, "prologue": 1.449e9 + 1.434e9}}
+MEASURED_TRAFFIC = {"720p-24B": {"core": 186.8e9 + 1.07e9, "prologue": 1.449e9 + 1.434e9,
+                                 "layer_norm": 1.0625e9 + 1.0619e9}}
 
 WORKLOADS = {
     # name: (T_lat frames per chunk, H, W, denoise chunks, prefix chunks, Hq, Hkv)
@@ -192,7 +193,7 @@ def cpu_baseline(inp, rows_per_chunk=6144):
                        f"{fl:.3e} FLOP in {dt:.1f} s (torch {torch.__version__} CPU SDPA fp32)"), o, idx
 
 
-def layer_norm_leg(inp, steps):
+def layer_norm_leg(inp, steps, traffic=None):
     """The LayerNorm of the layer input (the step ahead of the projections that feed the prologue), kernel-only:
     reported beside the headline, not part of `value`.  Re-uses the raw-q buffer as the hidden states and the
     cross-attention output buffer for the result (nothing reads that buffer afterwards)."""
@@ -213,7 +214,7 @@ def layer_norm_leg(inp, steps):
     ms = e0.elapsed_time(e1) / steps
     gbs = 2 * S * hidden * 2 / (ms * 1e-3) / 1e9
     return {"bound": "hbm", "kernel": "layer_norm_kernel", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS,
-            "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": None, "ms": round(ms, 4)}
+            "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": traffic, "ms": round(ms, 4)}
 
 
 def main():
@@ -288,7 +289,8 @@ def main():
     }
     if not args.no_fp8:
         result["fp8"] = fp8_leg(inp, core_fl, core_tflops, args.steps)
-    result["roofline_layer_norm"] = layer_norm_leg(inp, args.steps)
+    result["roofline_layer_norm"] = layer_norm_leg(inp, args.steps,
+                                                    MEASURED_TRAFFIC.get(args.workload, {}).get("layer_norm"))
     if args.copy_calibration:
         inp["xout"].copy_(inp["out"])  # reads and writes out.numel() * 2 bytes each
         torch.cuda.synchronize()

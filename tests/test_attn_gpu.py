@@ -428,8 +428,8 @@ def test_repeated_launches_are_bit_identical(dev):
 
 
 def test_graph_capture_and_replay(dev):
-    """The library allocates nothing, never synchronises and launches on the caller's stream, so a prologue +
-    attention pair can be captured into a HIP graph (the reference's enable_cuda_graph case).  Every replay, with
+    """The library allocates nothing, never synchronises and launches on the caller's stream, so an input norm +
+    prologue + attention sequence can be captured into a HIP graph (the reference's enable_cuda_graph case).  Every replay, with
     new inputs copied into the static buffers and eager work in between, must equal the eager result bit for bit."""
     S, Hq, Hkv, D, L = 3 * 96, 6, 2, 128, 96
     g = torch.Generator().manual_seed(11)
@@ -441,8 +441,11 @@ def test_graph_capture_and_replay(dev):
     kv = torch.empty(S, Hkv, 2 * D, dtype=torch.bfloat16, device=dev)
     out = torch.empty(S, Hq, D, dtype=torch.bfloat16, device=dev)
     tq, tk = _ranges(dev, O.q_ranges_for(3, L), O.default_kvrange(0, 3, L))
+    hid = mk(S, Hq * D)  # stands for the layer input; its norm feeds the q side here
+    w_ln, b_ln = mk(Hq * D), mk(Hq * D)
 
     def step(dst):
+        M.layer_norm(hid, w_ln, b_ln, 1e-6, out=q_raw)
         M.qk_prologue(q_raw, k_raw, v_raw, rope, z, z, z, z, Hq=Hq, Hkv=Hkv, kv_out=kv, n_cache_rows=S, q_out=q)
         M.range_attention(q, kv[..., :D], kv[..., D:], tq, tk, L, out=dst, return_lse=False)
 
@@ -455,7 +458,7 @@ def test_graph_capture_and_replay(dev):
     with torch.cuda.graph(graph):
         step(out)
     for rep in range(4):
-        for t in (q_raw, k_raw, v_raw):
+        for t in (hid, k_raw, v_raw):
             t.copy_(torch.randn(t.shape, generator=g).bfloat16())
         eager = torch.empty_like(out)
         step(eager)

@@ -689,18 +689,29 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   // ---- epilogue: normalise and store ----
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = 1.f / l_tot;
-  if (row_ok) {
-    char* op = a.out + (long)q_row * a.os_t + o_head;
+  // A lane holds four consecutive features per (mb, b), its partner in the other half wave the next four: the
+  // halves trade the odd-b registers of the lower half for the even-b registers of the upper one, after which
+  // every lane owns eight consecutive features and stores 16 bytes at a time.
+  // (the row address is derived here from an opaque copy of the lane index, or the compiler computes it at the
+  // top of the kernel and carries two more registers through the main loop, which the pre-scaled instantiations
+  // do not have)
+  int lane_e = l;
+  asm volatile("" : "+v"(lane_e));
+  char* const op = a.out + (long)(q0 + 32 * w + (lane_e & 31)) * a.os_t + o_head + 16 * (lane_e >> 5);
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+  for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int d = 32 * mb + 8 * b + 4 * g;
-        u32x2 pk;
-        pk[0] = pack_bf16x2(o_acc[mb][4 * b + 0] * inv, o_acc[mb][4 * b + 1] * inv);
-        pk[1] = pack_bf16x2(o_acc[mb][4 * b + 2] * inv, o_acc[mb][4 * b + 3] * inv);
-        *(u32x2*)(op + d * 2) = pk;
+    for (int bp = 0; bp < 2; ++bp) {
+      unsigned ev[2], od[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        ev[e] = pack_bf16x2(o_acc[mb][8 * bp + 2 * e] * inv, o_acc[mb][8 * bp + 2 * e + 1] * inv);
+        od[e] = pack_bf16x2(o_acc[mb][8 * bp + 4 + 2 * e] * inv, o_acc[mb][8 * bp + 4 + 2 * e + 1] * inv);
+        half_swap(ev[e], od[e]);  // lower half: (own even, partner's even); upper half: (partner's odd, own odd)
       }
+      if (row_ok) *(u32x4*)(op + (32 * mb + 16 * bp) * 2) = u32x4{ev[0], ev[1], od[0], od[1]};
+    }
+  if (row_ok) {
     if (a.lse && g == 0)
       a.lse[(long)h * a.total_q + q_row] = ((PRESC ? -neg_m[0] : m_run * c) + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   }

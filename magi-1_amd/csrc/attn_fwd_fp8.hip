@@ -424,18 +424,27 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   if (!wave_on) return;
   const float l_tot = l_run + __shfl_xor(l_run, 32);
   const float inv = v_max * __builtin_amdgcn_exp2f(-P_SHIFT) / l_tot;
-  if (row_ok) {
-    char* op = a.out + (long)q_row * a.os_t + o_head;
+  // A lane holds four consecutive features per (mb, b), its partner in the other half wave the next four: the
+  // halves trade the odd-b registers of the lower half for the even-b registers of the upper one, after which
+  // every lane owns eight consecutive features and stores 16 bytes at a time.  (The row address is derived from
+  // an opaque copy of the lane index so that it is computed here and not carried through the main loop.)
+  int lane_e = l;
+  asm volatile("" : "+v"(lane_e));
+  char* const op = a.out + (long)(q0 + 32 * w + (lane_e & 31)) * a.os_t + o_head + 16 * (lane_e >> 5);
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
+  for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) {
-        const int d = 32 * mb + 8 * b + 4 * g;
-        u32x2 pk;
-        pk[0] = pack_bf16x2(o_acc[mb][4 * b + 0] * inv, o_acc[mb][4 * b + 1] * inv);
-        pk[1] = pack_bf16x2(o_acc[mb][4 * b + 2] * inv, o_acc[mb][4 * b + 3] * inv);
-        *(u32x2*)(op + d * 2) = pk;
+    for (int bp = 0; bp < 2; ++bp) {
+      unsigned ev[2], od[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        ev[e] = pack_bf16x2(o_acc[mb][8 * bp + 2 * e] * inv, o_acc[mb][8 * bp + 2 * e + 1] * inv);
+        od[e] = pack_bf16x2(o_acc[mb][8 * bp + 4 + 2 * e] * inv, o_acc[mb][8 * bp + 4 + 2 * e + 1] * inv);
+        half_swap(ev[e], od[e]);  // lower half: (own even, partner's even); upper half: (partner's odd, own odd)
       }
+      if (row_ok) *(u32x4*)(op + (32 * mb + 16 * bp) * 2) = u32x4{ev[0], ev[1], od[0], od[1]};
+    }
+  if (row_ok) {
     if (a.lse && g == 0)
       a.lse[(long)h * a.total_q + q_row] = (m_run + __builtin_amdgcn_logf(l_tot)) * 0.6931471805599453f;
   }

@@ -15,6 +15,11 @@ __device__ __forceinline__ float half_swap_max(float x) {
   return fmaxf(lo, hi);
 }
 
+// Exchange lanes 32..63 of `a` with lanes 0..31 of `b` (both must be VALU results, see above).
+__device__ __forceinline__ void half_swap(unsigned& a, unsigned& b) {
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+}
+
 // max of three; written as nested fmaxf so that the compiler (which knows the wait states an MFMA result
 // needs before a VALU instruction may read it; it does not check inline assembly for them) forms v_max3_f32
 __device__ __forceinline__ float max3(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }

@@ -109,7 +109,7 @@ template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool PIPE = false, 
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
   constexpr int BM = 32 * NW;
   constexpr int TILE_BYTES = BN * ROW_BYTES;
-  constexpr int LW = NW > 8 ? 8 : NW;      // waves that load tiles (a 64-row tile is 16 loads of 4 rows)
+  constexpr int LW = NW > 8 ? 4 : NW;      // waves that load tiles (a 64-row tile is 16 loads of 4 rows); a multiple of 4
   constexpr int LOADS = BN / (4 * LW);     // direct loads per loading wave per matrix per tile (4 rows each)
   constexpr int WPS = NW * OCC / 4;        // waves per SIMD
   constexpr int TILE_LOADS = 2 * LOADS;    // ... per wave per tile

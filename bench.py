@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0
 Q_PREMUL = 128 ** -0.5 * math.log2(math.e)  # softmax_scale * log2(e) at head_dim 128
 # HBM-side bytes per launch on the 720p workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # plain copy of known size in the same run (FETCH_SIZE x2.0, WRITE_SIZE x1.0): profiles/bench_720p_hbm_traffic_pmc.txt
-MEASURED_TRAFFIC = {"720p-24B": {"core": 204e9 + 1.07e9, "prologue": 1.449e9 + 1.434e9,
+MEASURED_TRAFFIC = {"720p-24B": {"core": 195e9 + 1.07e9, "prologue": 1.449e9 + 1.434e9,
                                  "layer_norm": 1.0625e9 + 1.0619e9}}
 
 WORKLOADS = {

@@ -305,8 +305,10 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         for (int t = 0; t < 2; ++t) {
           s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[0], qf[0], neg_m, 0, 0, 0, e_k, 0, e_q);
           if (t == 0) ka[0] = read_k(1, 0);
+          __builtin_amdgcn_sched_barrier(0);  // (keeps each operand read one MFMA ahead of its use, where it is written)
           s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[1], qf[1], s_acc[t], 0, 0, 0, e_k, 0, e_q);
           if (t == 0) ka[1] = read_k(1, 1);
+          __builtin_amdgcn_sched_barrier(0);
         }
       } else {
 #pragma unroll

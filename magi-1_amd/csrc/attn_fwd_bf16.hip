@@ -25,13 +25,17 @@
 //     buffered, ONE V slot that is refilled under the score MFMAs and the softmax of the same tile,
 //     two barriers per tile, slots named statically): small grids and short key ranges;
 //   * 12 waves per workgroup (DB), ONE workgroup per CU, 64 KB of LDS (K and V double buffered in
-//     four statically named slots, one barrier per tile): every K / V tile is fetched from L2 once
+//     four statically named slots, one barrier per tile, the tile loads issued by four of the
+//     waves, one per SIMD): every K / V tile is fetched from L2 once
 //     for 384 query rows instead of 128.  On grids of many rounds with long key ranges this is the
 //     faster one, although it needs more cycles: the part is power limited, and the bytes it does
 //     not move come back as clock.
 // Both have a PRESC form that takes q already multiplied by softmax_scale * log2(e) (the prologue
 // does that ahead of q's rounding to bf16) and accumulates the score MFMAs onto the negated running
 // maximum, so the MFMA result is the exp2 argument and no per-score multiply-subtract remains.
+// Operand reads from LDS are written a few MFMAs ahead of their use and held there with scheduling
+// barriers (the instruction scheduler otherwise sinks them to one MFMA ahead); the epilogue trades
+// registers between the half waves so that every lane stores 16 contiguous bytes.
 // Instantiations with 2 waves / SIMD (deep prefetch, K and V double buffered), with 32-key tiles,
 // with 8-wave workgroups, and a software-pipelined loop (PIPE: score MFMAs of the next tile, softmax
 // and PV MFMAs of the current one interleaved in one basic block, 2 waves / SIMD) are kept for

@@ -119,14 +119,14 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.n_ranges = p->n_ranges;
   a.ranges_mode = p->ranges_mode;
   // q rows per workgroup.  bf16: 384 (12 waves, one workgroup per CU, every K / V tile fetched once for three
-  // times as many rows and one barrier per tile) pays on grids of many rounds with long key ranges; its coarser
-  // q tiles and longer jobs cost more than that on small grids and on short key ranges (cross attention), which
-  // keep 128 (4 waves, three workgroups per CU).
+  // times as many rows and one barrier per tile) pays on grids of many rounds with long key ranges (measured: +3 %
+  // at 43 rounds, +1 % at 9.4, -3 % at 5.3); its coarser q tiles and longer jobs cost more than that on small
+  // grids and on short key ranges (cross attention), which keep 128 (4 waves, three workgroups per CU).
   a.block_m = 128;
   if (p->dtype == MAGI_DTYPE_BF16) {
     const double wg384 = (double)p->Hq * p->n_ranges * ((p->max_seqlen_q + 383) / 384);
     const bool long_keys = p->max_seqlen_k == 0 || p->max_seqlen_k >= 4096;  // (0 = not stated)
-    if (wg384 >= 24.0 * compute_units() && long_keys) a.block_m = 384;
+    if (wg384 >= 9.0 * compute_units() && long_keys) a.block_m = 384;
     if (const char* e = std::getenv("MAGI_ATTN_BLOCK_M")) {  // tuning knob: 128, 256 or 384
       const int v = std::atoi(e);
       if (v == 128 || v == 256 || v == 384) a.block_m = v;

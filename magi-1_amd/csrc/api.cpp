@@ -225,8 +225,9 @@ int magi_layer_norm(const void* x, int64_t x_stride, const void* weight, const v
   if (x_stride % 8 || y_stride % 8 || !aligned16(x) || !aligned16(y))
     return fail(MAGI_EINVAL, "magi_layer_norm: rows must be 16-byte aligned");
   if (!(eps >= 0.f)) return fail(MAGI_EINVAL, "magi_layer_norm: eps");
+  if (rows > 0x7fffffffLL * 4) return fail(MAGI_ENOSYS, "magi_layer_norm: more than 2^33 rows");  // (4 rows per workgroup)
   hipError_t e = magi::launch_layer_norm(static_cast<const char*>(x), x_stride * 2, weight, bias, params_fp32 != 0,
-                                         static_cast<char*>(y), y_stride * 2, rows, cols, eps, compute_units(),
+                                         static_cast<char*>(y), y_stride * 2, rows, cols, eps,
                                          static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_layer_norm launch");
   return MAGI_OK;

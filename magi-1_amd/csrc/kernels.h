@@ -63,7 +63,7 @@ hipError_t launch_prologue(const PrologueKernArgs& a, hipStream_t stream);
 hipError_t launch_head_norm(const char* x, long x_stride_t, long x_stride_h, const float* gamma, const float* beta,
                             char* y, int S, int H, int norm_kind, float eps, hipStream_t stream);
 hipError_t launch_layer_norm(const char* x, long x_stride, const void* w, const void* b, int params_fp32, char* y,
-                             long y_stride, long rows, int cols, float eps, int compute_units, hipStream_t stream);
+                             long y_stride, long rows, int cols, float eps, hipStream_t stream);
 hipError_t launch_rotary(const void* x, const float* cos, const float* sin, void* y, int B, int S, int H, int D,
                          int R2, int is_bf16, hipStream_t stream);
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,

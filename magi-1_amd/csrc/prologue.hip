@@ -192,88 +192,98 @@ __global__ __launch_bounds__(THREADS) void head_norm_kernel(const char* x, long 
   *(u32x4*)(dst + eb * 2) = pack8(v + 8);
 }
 
-// Row LayerNorm of the layer input: one wavefront per row, the row held in registers as NV 16-byte
-// vectors per lane (vector i of lane l covers elements (64 i + l) * 8 ...), fp32 statistics in two
-// passes over the registers, weight and bias staged once per workgroup in LDS as fp32.  A workgroup
-// walks rows with a grid stride so the parameters are staged once per resident workgroup.
-constexpr int LN_THREADS = 512;  // 8 rows in flight per workgroup share one staged copy of the parameters
-
-template <int NV>
-__global__ __launch_bounds__(LN_THREADS) void layer_norm_kernel(const char* x, long xs, const void* w, const void* b,
-                                                             int params_fp32, char* y, long ys, long rows, int cols,
-                                                             float eps) {
-  // four planes [cols / 8][4]: weight elements 0-3 and 4-7 of every group of eight, then the bias likewise, so
-  // that a lane's 16-byte reads are 16 bytes apart from its neighbours' (no bank conflicts)
-  extern __shared__ __attribute__((aligned(16))) float s_wb[];
+// Row LayerNorm of the layer input: one wavefront per row, the row held packed in registers as NV 16-byte
+// vectors per lane (vector i of lane l covers elements (64 i + l) * 8 ...), fp32 statistics in two passes over
+// the registers.  Weight and bias are read straight from global memory in the last pass (they stay in L1 / L2);
+// a persistent variant that staged them in LDS once per workgroup measured 7-8 % slower.
+template <int NV, bool PF32>
+__global__ __launch_bounds__(THREADS) void layer_norm_kernel(const char* x, long xs, const char* w, const char* b,
+                                                             char* y, long ys, long rows, int cols, float eps) {
   const int tid = threadIdx.x;
-  const int plane = cols >> 1;  // floats per plane
-  for (int i = tid; i < 2 * cols; i += LN_THREADS) {
-    const void* src = i < cols ? w : b;
-    const int e = i < cols ? i : i - cols;
-    float v = i < cols ? 1.f : 0.f;
-    if (src) {
-      v = params_fp32 ? ((const float*)src)[e]
-                      : __builtin_bit_cast(float, (unsigned)((const unsigned short*)src)[e] << 16);
-    }
-    s_wb[(i < cols ? 0 : 2 * plane) + ((e >> 2) & 1) * plane + (e >> 3) * 4 + (e & 3)] = v;
-  }
-  __syncthreads();
   const int lane = tid & 63;
   const int nvec = cols >> 3;
   const float inv_n = 1.f / (float)cols;
-  const long step = (long)gridDim.x * (LN_THREADS / 64);
-  for (long row = (long)blockIdx.x * (LN_THREADS / 64) + (tid >> 6); row < rows; row += step) {
-    const char* src = x + row * xs;
-    u32x4 raw[NV];
+  const long row = (long)blockIdx.x * (THREADS / 64) + (tid >> 6);
+  if (row >= rows) return;
+  const char* src = x + row * xs;
+  u32x4 raw[NV];
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      const int vi = i * 64 + lane;
-      raw[i] = vi < nvec ? *(const u32x4*)(src + (long)vi * 16) : u32x4{0u, 0u, 0u, 0u};
-    }
-    float s = 0.f;
+  for (int i = 0; i < NV; ++i) {
+    const int vi = i * 64 + lane;
+    raw[i] = vi < nvec ? *(const u32x4*)(src + (long)vi * 16) : u32x4{0u, 0u, 0u, 0u};
+  }
+  float s = 0.f;
 #pragma unroll
-    for (int i = 0; i < NV; ++i) {
+  for (int i = 0; i < NV; ++i) {
+    float f[8];
+    unpack8(raw[i], f);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) s += f[k];
+  }
+  const float mean = wave_sum(s) * inv_n;
+  // the row stays packed between the passes (48 registers for 6144 columns instead of 96 more for its fp32
+  // form): the empty asm makes the compiler unpack again rather than keep the first pass's values
+#pragma unroll
+  for (int i = 0; i < NV; ++i) asm volatile("" : "+v"(raw[i]));
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    if (i * 64 + lane < nvec) {
       float f[8];
       unpack8(raw[i], f);
 #pragma unroll
-      for (int k = 0; k < 8; ++k) s += f[k];
-    }
-    const float mean = wave_sum(s) * inv_n;
-    // the row stays packed between the passes (48 registers for 6144 columns instead of 96 more for its fp32
-    // form): the empty asm makes the compiler unpack again rather than keep the first pass's values
-#pragma unroll
-    for (int i = 0; i < NV; ++i) asm volatile("" : "+v"(raw[i]));
-    float q = 0.f;
-#pragma unroll
-    for (int i = 0; i < NV; ++i) {
-      if (i * 64 + lane < nvec) {
-        float f[8];
-        unpack8(raw[i], f);
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-          const float d = f[k] - mean;
-          q += d * d;
-        }
+      for (int k = 0; k < 8; ++k) {
+        const float d = f[k] - mean;
+        q += d * d;
       }
     }
-    const float rstd = __builtin_amdgcn_rsqf(wave_sum(q) * inv_n + eps);
+  }
+  const float rstd = __builtin_amdgcn_rsqf(wave_sum(q) * inv_n + eps);
 #pragma unroll
-    for (int i = 0; i < NV; ++i) asm volatile("" : "+v"(raw[i]));
-    char* dst = y + row * ys;
+  for (int i = 0; i < NV; ++i) asm volatile("" : "+v"(raw[i]));
+  char* dst = y + row * ys;
+  auto param8 = [&](const char* p, int vi, float* out) {  // elements 8 vi .. 8 vi + 7 of a parameter
+    if (PF32) {
+      const f32x4 lo = *(const f32x4*)(p + (long)vi * 32), hi = *(const f32x4*)(p + (long)vi * 32 + 16);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        out[k] = lo[k];
+        out[4 + k] = hi[k];
+      }
+    } else {
+      unpack8(*(const u32x4*)(p + (long)vi * 16), out);
+    }
+  };
+  if (w && b) {  // the usual case, free of branches so that the parameter loads of all vectors go out together
 #pragma unroll
     for (int i = 0; i < NV; ++i) {
       const int vi = i * 64 + lane;
       if (vi < nvec) {
-        float f[8];
+        float f[8], wf[8], bf[8];
         unpack8(raw[i], f);
-        const f32x4* par = (const f32x4*)s_wb + vi;
-        const int pv = plane >> 2;  // 16-byte vectors per plane
-        const f32x4 w0 = par[0], w1 = par[pv], b0 = par[2 * pv], b1 = par[3 * pv];
+        param8(w, vi, wf);
+        param8(b, vi, bf);
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-          f[k] = (f[k] - mean) * rstd * w0[k] + b0[k];
-          f[k + 4] = (f[k + 4] - mean) * rstd * w1[k] + b1[k];
+        for (int k = 0; k < 8; ++k) f[k] = (f[k] - mean) * rstd * wf[k] + bf[k];
+        *(u32x4*)(dst + (long)vi * 16) = pack8(f);
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int vi = i * 64 + lane;
+      if (vi < nvec) {
+        float f[8], wf[8], bf[8];
+        unpack8(raw[i], f);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+          wf[k] = 1.f;
+          bf[k] = 0.f;
         }
+        if (w) param8(w, vi, wf);
+        if (b) param8(b, vi, bf);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) f[k] = (f[k] - mean) * rstd * wf[k] + bf[k];
         *(u32x4*)(dst + (long)vi * 16) = pack8(f);
       }
     }
@@ -346,16 +356,21 @@ hipError_t launch_head_norm(const char* x, long x_stride_t, long x_stride_h, con
 }
 
 hipError_t launch_layer_norm(const char* x, long x_stride, const void* w, const void* b, int params_fp32, char* y,
-                             long y_stride, long rows, int cols, float eps, int compute_units, hipStream_t stream) {
+                             long y_stride, long rows, int cols, float eps, hipStream_t stream) {
   if (rows <= 0) return hipSuccess;
   const int need = (cols / 8 + 63) / 64;  // 16-byte vectors per lane
-  const size_t lds = (size_t)2 * cols * sizeof(float);
-  const long wgs = (rows + LN_THREADS / 64 - 1) / (LN_THREADS / 64);
-  const long resident = (long)compute_units * 4;
-  const dim3 grid((unsigned)(wgs < resident ? wgs : resident)), block(LN_THREADS);
-#define MAGI_LN(NV)                                                                                              \
-  hipLaunchKernelGGL(layer_norm_kernel<NV>, grid, block, lds, stream, x, x_stride, w, b, params_fp32, y, y_stride, \
-                     rows, cols, eps)
+  const dim3 grid((unsigned)((rows + THREADS / 64 - 1) / (THREADS / 64))), block(THREADS);
+  const char* wp = static_cast<const char*>(w);
+  const char* bp = static_cast<const char*>(b);
+#define MAGI_LN(NV)                                                                                               \
+  do {                                                                                                            \
+    if (params_fp32)                                                                                              \
+      hipLaunchKernelGGL((layer_norm_kernel<NV, true>), grid, block, 0, stream, x, x_stride, wp, bp, y, y_stride, \
+                         rows, cols, eps);                                                                        \
+    else                                                                                                          \
+      hipLaunchKernelGGL((layer_norm_kernel<NV, false>), grid, block, 0, stream, x, x_stride, wp, bp, y,          \
+                         y_stride, rows, cols, eps);                                                              \
+  } while (0)
   if (need <= 2) MAGI_LN(2);
   else if (need <= 4) MAGI_LN(4);
   else if (need <= 6) MAGI_LN(6);

@@ -89,7 +89,24 @@ const char* magi_last_error(void);
  * q_scale,k_scale,v_scale  fp8 only: DEVICE fp32 [n_scale_chunks, H] with the scale of token t
  *                        at [t / scale_chunk_tokens, h]; NULL for bf16
  * softmax_scale          <= 0 selects D^-0.5
+ * score_bound            0 = unknown.  > 0 (bf16 with MAGI_ATTN_Q_PRESCALED only): the caller's promise that every
+ *                        score satisfies |q . k| <= score_bound, in the units q was pre-scaled to (exp2 exponents).
+ *                        Up to MAGI_SCORE_BOUND_MAX the softmax is then evaluated as 2^score / sum 2^score without a
+ *                        running maximum (it is shift invariant, and 2^score can neither overflow nor lose its
+ *                        leading terms in fp32 at such bounds): the same result with a third fewer vector
+ *                        instructions, and room for kernels that hold 64 query rows per wavefront.  QK-normed
+ *                        attention knows the bound from its norm parameters:
+ *                        |q| |k| <= (sqrt(D) max|gamma_q + 1| + |beta_q|) (sqrt(D) max|gamma_k + 1| + |beta_k|),
+ *                        times the pre-scale factor.  Larger bounds fall back to the running maximum.  A promise
+ *                        that does not hold gives inf / nan or wrong rows, not a fault.  No counterpart in the
+ *                        reference.
+ * q_tile_rows            0 = the library picks the workgroup shape from the size of the launch.  Otherwise the
+ *                        number of query rows per workgroup to use: 128 or 384 (bf16), 256 or 512 (bf16 with a
+ *                        score_bound in force), 128 (fp8); anything else is MAGI_EINVAL.  Results do not depend on
+ *                        it beyond the order of fp32 additions; it exists so that every shipped workgroup shape
+ *                        can be exercised on small inputs.
  */
+#define MAGI_SCORE_BOUND_MAX 64.0f
 typedef struct magi_attn_args {
   const void* q;
   const void* k;
@@ -117,6 +134,8 @@ typedef struct magi_attn_args {
   int32_t flags; /* MAGI_ATTN_* bits */
   int32_t out_group_heads;
   int64_t o_stride_g;
+  float score_bound;
+  int32_t q_tile_rows;
 } magi_attn_args;
 
 int magi_attn_fwd(const magi_attn_args* args, void* stream);

@@ -40,11 +40,20 @@ int compute_units() {
   return cached[dev];
 }
 
+#ifdef MAGI_TUNING
+// Tuning builds only (make TUNING=1): MAGI_ATTN_BLOCK_M / MAGI_ATTN_VARIANT pick a bf16 kernel instantiation by hand
+// for A/B measurements.  Read once per process; the shipped library has no such knobs.
+int tuning_env(const char* name) {
+  const char* e = std::getenv(name);
+  return e ? std::atoi(e) : 0;
+}
+#endif
+
 }  // namespace
 
 extern "C" {
 
-int magi_version(void) { return 100; }
+int magi_version(void) { return 101; }
 
 const char* magi_last_error(void) { return g_err; }
 
@@ -75,6 +84,18 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     return fail(MAGI_EINVAL, "magi_attn_fwd: q/k/v/out must be 16-byte aligned");
   if (p->q_stride_h < p->D || p->k_stride_h < p->D || p->v_stride_h < p->D || p->o_stride_h < p->D)
     return fail(MAGI_EINVAL, "magi_attn_fwd: head stride smaller than head_dim");
+  if (p->q_stride_t < p->D || p->k_stride_t < p->D || p->v_stride_t < p->D || p->o_stride_t < p->D)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: token stride smaller than head_dim (rows may not overlap or run backwards)");
+  // (the kernels address a 64-key tile with 32-bit byte offsets from its first row)
+  if (p->k_stride_t > (1 << 23) || p->v_stride_t > (1 << 23))
+    return fail(MAGI_ENOSYS, "magi_attn_fwd: k / v token strides above 2^23 elements are not implemented");
+  if (p->dtype == MAGI_DTYPE_FP8_E4M3 && (p->flags & MAGI_ATTN_Q_PRESCALED))
+    return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_Q_PRESCALED is a bf16 flag (fp8: MAGI_ATTN_FP8_POW2_PRESCALED)");
+  if (p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_FP8_POW2_PRESCALED))
+    return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_FP8_POW2_PRESCALED is an fp8 flag");
+  if (!(p->score_bound >= 0.f)) return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound must be >= 0");
+  if (p->score_bound > 0.f && !(p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)))
+    return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound needs bf16 inputs with MAGI_ATTN_Q_PRESCALED");
   if (p->out_group_heads < 0 || (p->out_group_heads > 0 && (p->Hq % p->out_group_heads || p->o_stride_g % 8)))
     return fail(MAGI_EINVAL, "magi_attn_fwd: out_group_heads must divide Hq and o_stride_g keep rows 16-byte aligned");
   int k_split = p->total_k;
@@ -118,27 +139,42 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.k_split = k_split;
   a.n_ranges = p->n_ranges;
   a.ranges_mode = p->ranges_mode;
-  // q rows per workgroup.  bf16: 384 (12 waves, one workgroup per CU, every K / V tile fetched once for three
-  // times as many rows and one barrier per tile) pays on grids of many rounds with long key ranges (measured: +3 %
-  // at 43 rounds, +1 % at 9.4, -3 % at 5.3); its coarser q tiles and longer jobs cost more than that on small
-  // grids and on short key ranges (cross attention), which keep 128 (4 waves, three workgroups per CU).
+  // Kernel choice for bf16.
+  //  * Scores with a promised bound (score_bound): the kernel without a running maximum that holds 64 query rows per
+  //    wavefront (every K / V fragment read from LDS feeds two MFMAs); 256-row workgroups (4 waves, two per CU).
+  //  * Otherwise 32 rows per wavefront with the online softmax: 384-row workgroups (12 waves, one workgroup per CU,
+  //    every K / V tile fetched once for three times as many rows and one barrier per tile) pay on grids of many
+  //    rounds with long key ranges (measured: +3 % at 43 rounds, +1 % at 9.4, -3 % at 5.3); small grids and short
+  //    key ranges (cross attention) keep 128 rows (4 waves, three workgroups per CU).
   a.block_m = 128;
+  if (p->dtype == MAGI_DTYPE_FP8_E4M3 && p->q_tile_rows != 0 && p->q_tile_rows != 128)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (fp8: 128)", p->q_tile_rows);
+  const bool bounded = p->dtype == MAGI_DTYPE_BF16 && p->score_bound > 0.f && p->score_bound <= MAGI_SCORE_BOUND_MAX;
   if (p->dtype == MAGI_DTYPE_BF16) {
     const double wg384 = (double)p->Hq * p->n_ranges * ((p->max_seqlen_q + 383) / 384);
     const bool long_keys = p->max_seqlen_k == 0 || p->max_seqlen_k >= 4096;  // (0 = not stated)
-    if (wg384 >= 9.0 * compute_units() && long_keys) a.block_m = 384;
-    if (const char* e = std::getenv("MAGI_ATTN_BLOCK_M")) {  // tuning knob: 128, 256 or 384
-      const int v = std::atoi(e);
-      if (v == 128 || v == 256 || v == 384) a.block_m = v;
+    if (bounded)
+      a.block_m = (wg384 >= 9.0 * compute_units() && long_keys) ? 512 : 256;
+    else if (wg384 >= 9.0 * compute_units() && long_keys)
+      a.block_m = 384;
+    if (p->q_tile_rows != 0) {
+      const int r = p->q_tile_rows;
+      if (bounded ? (r != 256 && r != 512) : (r != 128 && r != 384))
+        return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (bf16: 128 or 384; with a score bound: 256 or 512)", r);
+      a.block_m = r;
     }
+#ifdef MAGI_TUNING
+    static const int env_block_m = tuning_env("MAGI_ATTN_BLOCK_M"), env_variant = tuning_env("MAGI_ATTN_VARIANT");
+    if (env_block_m == 128 || env_block_m == 256 || env_block_m == 384 || env_block_m == 512) a.block_m = env_block_m;
+    a.variant = env_variant;
+#endif
   }
-  if (const char* e = std::getenv("MAGI_ATTN_VARIANT")) a.variant = std::atoi(e);  // tuning knob
   a.tiles_per_range = (p->max_seqlen_q + a.block_m - 1) / a.block_m;
   a.Hq = p->Hq;
   a.Hkv = p->Hkv;
   a.G = p->Hq / p->Hkv;
   a.scale_chunk_tokens = p->scale_chunk_tokens;
-  a.flags = p->flags;
+  a.flags = p->flags | (bounded ? magi::ATTN_BOUNDED : 0);
   const double total = (double)p->Hq * p->n_ranges * a.tiles_per_range;
   if (total > 2.0e9) return fail(MAGI_EINVAL, "magi_attn_fwd: grid too large (%.3g workgroups)", total);
   a.total_wgs = (unsigned)total;
@@ -147,8 +183,13 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.scale_log2 = scale * 1.4426950408889634f;
   if (p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)) a.scale_log2 = 1.f;  // q . k is the exp2 exponent
 
-  hipError_t e = p->dtype == MAGI_DTYPE_BF16 ? magi::launch_attn_fwd_bf16(a, static_cast<hipStream_t>(stream))
-                                             : magi::launch_attn_fwd_fp8(a, static_cast<hipStream_t>(stream));
+  hipError_t e;
+  if (p->dtype != MAGI_DTYPE_BF16)
+    e = magi::launch_attn_fwd_fp8(a, static_cast<hipStream_t>(stream));
+  else if (bounded || a.variant >= 10)
+    e = magi::launch_attn_fwd_bf16_w64(a, static_cast<hipStream_t>(stream));
+  else
+    e = magi::launch_attn_fwd_bf16(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_attn_fwd launch");
   return MAGI_OK;
 }

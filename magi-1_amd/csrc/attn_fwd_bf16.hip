@@ -742,23 +742,32 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  if (a.block_m == 384 && (a.flags & 2) && a.variant != 7)  // ... q pre-scaled: scores are exp2 exponents (PRESC)
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true, true>), dim3(grid), dim3(768), 0, stream, a);
-  else if (a.block_m == 384)  // 12 waves, 384 query rows, one workgroup per CU = 3 waves / SIMD sharing every tile
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true>), dim3(grid), dim3(768), 0, stream, a);
-  else if (a.block_m == 256 && a.variant == 3)  // software-pipelined loop, 8 waves, 256 query rows, 2 waves / SIMD
+  const bool presc = (a.flags & 2) != 0;  // q pre-scaled: the scores are exp2 exponents (PRESC instantiations)
+#ifdef MAGI_TUNING
+  // comparison instantiations, reachable in tuning builds only (MAGI_ATTN_BLOCK_M / MAGI_ATTN_VARIANT)
+  if (a.block_m == 256 && a.variant == 3)  // software-pipelined loop, 8 waves, 256 query rows, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false, true>), dim3(grid), dim3(512), 0, stream, a);
   else if (a.block_m == 256)  // 8 waves, 256 query rows, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false>), dim3(grid), dim3(512), 0, stream, a);
-  else if (a.variant == 1)  // 32-key tiles, 3-stage ring, 3 waves / SIMD
+  else if (a.block_m == 128 && a.variant == 1)  // 32-key tiles, 3-stage ring, 3 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 32, 3, 3, false>), dim3(grid), dim3(256), 0, stream, a);
-  else if (a.variant == 2)  // 64-key tiles, double-buffered K and V, 2 waves / SIMD
+  else if (a.block_m == 128 && a.variant == 2)  // 64-key tiles, double-buffered K and V, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false>), dim3(grid), dim3(256), 0, stream, a);
-  else if (a.variant == 3)  // software-pipelined loop, 2 waves / SIMD
+  else if (a.block_m == 128 && a.variant == 3)  // software-pipelined loop, 2 waves / SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false, true>), dim3(grid), dim3(256), 0, stream, a);
-  else if ((a.flags & 2) && a.variant != 7)  // 4 waves, q pre-scaled (PRESC)
+  else if (a.block_m == 384 && a.variant == 7)  // pre-scaled q through the instantiation with the per-score multiply
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true>), dim3(grid), dim3(768), 0, stream, a);
+  else if (a.variant == 7)
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), dim3(grid), dim3(256), 0, stream, a);
+  else
+#endif
+  if (a.block_m == 384 && presc)  // 12 waves, 384 query rows, one workgroup per CU = 3 waves / SIMD sharing every tile
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true, true>), dim3(grid), dim3(768), 0, stream, a);
+  else if (a.block_m == 384)
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true>), dim3(grid), dim3(768), 0, stream, a);
+  else if (presc)  // 4 waves, 64-key tiles, double-buffered K, single V slot, three workgroups per CU
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true, false, false, true>), dim3(grid), dim3(256), 0, stream, a);
-  else  // 4 waves, 64-key tiles, double-buffered K, single V slot, three workgroups per CU
+  else
     hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), dim3(grid), dim3(256), 0, stream, a);
   return hipGetLastError();
 }

@@ -166,7 +166,6 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   };
   const unsigned kvoff = (unsigned)row_in_tile0 * (unsigned)ks_t + (unsigned)(kchunk * 16);
   const unsigned vvoff = (unsigned)row_in_tile0 * (unsigned)vs_t + (unsigned)(vchunk * 16);
-  const bool small_strides = ks_t * (BN + 8) < (1l << 31) && vs_t * (BN + 8) < (1l << 31);
   const char* const kcol_u = a.k + (long)kvh * a.ks_h;  // wave-uniform column bases
   const char* const vcol_u = a.v + (long)kvh * a.vs_h;
   auto issue_tile = [&](int k0, int pe, auto BUFC) {
@@ -174,7 +173,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
     unsigned char* const dK = BUF ? sK1 : sK0;
     unsigned char* const dV = BUF ? sV1 : sV0;
     const bool second = k0 >= k_split;
-    if (small_strides && k0 + BN <= pe) {
+    if (k0 + BN <= pe) {
       // full tile inside one piece: buffer-addressed direct loads (scalar base in the descriptor, one
       // loop-invariant 32-bit lane offset, the row group in the scalar offset) cost the SIMD next to nothing
       // to issue, unlike the same load with a 64-bit address per lane
@@ -191,15 +190,20 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       }
       return;
     }
-    const char* kb = kcolp + (second ? k2_delta : 0);
-    const char* vb = vcolp + (second ? v2_delta : 0);
+    // ragged end of a piece: per-lane rows clamped to the piece's last key.  Still buffer loads: a global_load ... lds
+    // anywhere in the kernel counts as a possible FLAT access to LDS, after which the compiler waits for ALL
+    // outstanding LDS reads in front of every MFMA instead of counting them.
+    const __amdgpu_buffer_rsrc_t kr = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(kcol_u + (long)k0 * ks_t + (second ? k2_delta : 0)), 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t vr = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(vcol_u + (long)k0 * vs_t + (second ? v2_delta : 0)), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
-      const int row = min(k0 + row_in_tile0 + 8 * NW * j, pe - 1);
-      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(kb + (long)row * ks_t), LDS_PTR(void, dK + (w + j * NW) * 1024),
-                                       16, 0, 0);
-      __builtin_amdgcn_global_load_lds(GLOBAL_PTR(vb + (long)row * vs_t), LDS_PTR(void, dV + (w + j * NW) * 1024),
-                                       16, 0, 0);
+      const int rel = min(row_in_tile0 + 8 * NW * j, pe - 1 - k0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, LDS_PTR(void, dK + (w + j * NW) * 1024), 16,
+                                               (unsigned)rel * (unsigned)ks_t + (unsigned)(kchunk * 16), 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, LDS_PTR(void, dV + (w + j * NW) * 1024), 16,
+                                               (unsigned)rel * (unsigned)vs_t + (unsigned)(vchunk * 16), 0, 0, 0);
     }
   };
 

@@ -24,17 +24,21 @@ struct AttnKernArgs {
   int out_group; // heads per output group, 0 = heads addressed by os_h alone
   int total_q, total_k, k_split;
   int n_ranges, ranges_mode, tiles_per_range;
-  int block_m;  // q rows per workgroup: 128 (4 waves) or 256 (8 waves)
-  int variant;  // bf16 kernel instantiation, see launch_attn_fwd_bf16 (0 = default)
+  int block_m;  // q rows per workgroup (the launchers map it to an instantiation)
+  int variant;  // tuning builds: bf16 kernel instantiation picked by hand (0 = the library's own choice)
   int Hq, Hkv, G;
   int scale_chunk_tokens;
-  int flags;
+  int flags;  // MAGI_ATTN_* bits of the public header, plus ATTN_BOUNDED
   unsigned total_wgs, per_xcd;
   float scale_log2;  // softmax_scale * log2(e)
 };
 
 
+// internal flag: the caller promised bounded scores (magi_attn_args.score_bound within MAGI_SCORE_BOUND_MAX)
+constexpr int ATTN_BOUNDED = 1 << 8;
+
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream);
+hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream);
 hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream);
 
 struct PrologueKernArgs {

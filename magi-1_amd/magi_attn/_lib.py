@@ -20,6 +20,7 @@ MAGI_NORM_RMSNORM_1P = 1
 MAGI_NORM_NONE = 2
 MAGI_ATTN_FP8_POW2_PRESCALED = 1
 MAGI_ATTN_Q_PRESCALED = 2
+MAGI_SCORE_BOUND_MAX = 64.0
 
 
 class MagiError(RuntimeError):
@@ -43,7 +44,8 @@ class AttnArgs(C.Structure):
         ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32),
         ("dtype", C.c_int32), ("scale_chunk_tokens", C.c_int32),
         ("softmax_scale", C.c_float), ("flags", C.c_int32),
-        ("out_group_heads", C.c_int32), ("o_stride_g", C.c_int64),
+        ("out_group_heads", C.c_int32), ("o_stride_g", C.c_int64), ("score_bound", C.c_float),
+        ("q_tile_rows", C.c_int32),
     ]
 
 

@@ -67,6 +67,8 @@ def range_attention(
     scale_chunk_tokens: int = 0,
     fp8_pow2_prescaled: bool = False,
     q_prescaled: bool = False,
+    score_bound: float = 0.0,
+    q_tile_rows: int = 0,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = True,
     zero_init: bool = True,
@@ -78,6 +80,9 @@ def range_attention(
 
     q_prescaled (bf16): q already carries softmax_scale * log2(e) (qk_prologue(..., q_premul=that)), so q . k is the
     exp2 exponent: the kernel skips its per-score multiply; softmax_scale is ignored.
+
+    score_bound (with q_prescaled): promise that |q . k| <= score_bound for every pair; see magi_attn_args.score_bound.
+    q_tile_rows: force a workgroup shape (0 = the library's choice); see magi_attn_args.q_tile_rows.
     """
     _check_thd(q, "q")
     _check_thd(k, "k")
@@ -134,6 +139,8 @@ def range_attention(
     a.scale_chunk_tokens = int(scale_chunk_tokens)
     a.softmax_scale = 0.0 if softmax_scale is None else float(softmax_scale)
     a.flags = (L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0) | (L.MAGI_ATTN_Q_PRESCALED if q_prescaled else 0)
+    a.score_bound = float(score_bound)
+    a.q_tile_rows = int(q_tile_rows)
     with torch.cuda.device(q.device):
         L.check(L.lib().magi_attn_fwd(C.byref(a), _stream()))
     return out, lse

@@ -1,0 +1,155 @@
+"""GPU parity of the bounded-score attention path (64 query rows per wavefront, no running maximum; through
+the C-ABI with magi_attn_args.score_bound) against the CPU oracle and against the online-softmax kernel.
+
+The inputs are what the layer produces: q pre-multiplied by softmax_scale * log2(e) before its one rounding to
+bf16, per-head normalised q and k, so that |q . k| <= |q| |k| is known.  Tolerance as for the other bf16 tests
+(benchmark definition): max-abs <= 2e-2 and cosine >= 0.9999 against the fp32 reference."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import magi_attn as M
+from oracle import magi_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+MAX_ABS = 2e-2
+MIN_COS = 0.9999
+PREMUL = 128 ** -0.5 * math.log2(math.e)
+LN2 = math.log(2.0)
+
+
+def _cmp(out, ref, what=""):
+    o = out.detach().double().cpu().flatten()
+    r = ref.detach().double().cpu().flatten()
+    err = (o - r).abs().max().item()
+    cos = (torch.dot(o, r) / (o.norm() * r.norm()).clamp_min(1e-30)).item()
+    assert err <= MAX_ABS, f"{what}: max-abs {err}"
+    assert cos >= MIN_COS, f"{what}: cosine {cos}"
+    return err, cos
+
+
+def _ranges(dev, *arrs):
+    return [torch.tensor(np.asarray(a), dtype=torch.int32, device=dev) for a in arrs]
+
+
+def _inputs(Tq, Tk, Hq, Hkv, seed, gain=1.0):
+    """q (pre-scaled, bf16), k, v and the Cauchy-Schwarz bound of |q . k| computed from the tensors themselves."""
+    q, k, v = O.synthetic_qkv(Tq, Tk, Hq, Hkv, 128, seed=seed, dtype=torch.float32)
+    q = (q * (gain * PREMUL)).bfloat16()
+    k = (k * gain).bfloat16()
+    v = v.bfloat16()
+    bound = (q.float().norm(dim=-1).max() * k.float().norm(dim=-1).max()).item() if Tk else 1.0
+    return q, k, v, bound
+
+
+CASES = [
+    # L, dn, sp, Hq, Hkv
+    (128, 1, 0, 1, 1),      # half a q tile of the 256-row workgroup, two key tiles
+    (64, 2, 0, 2, 1),       # one wave of the four
+    (200, 3, 1, 6, 2),      # ragged everywhere, GQA 3
+    (77, 2, 2, 3, 1),       # L below one tile; second row block of wave 1 partly filled
+    (1, 3, 2, 6, 1),        # single-token chunks, GQA 6
+    (333, 4, 3, 12, 4),     # two q tiles per range, 13 rows in the last wave
+    (1536, 3, 0, 24, 8),    # the CPU-runnable benchmark configuration
+]
+
+
+@pytest.mark.parametrize("rows", [0, 256, 512])
+@pytest.mark.parametrize("L,dn,sp,Hq,Hkv", CASES)
+def test_bounded_chunk_causal_parity(dev, L, dn, sp, Hq, Hkv, rows):
+    """rows: the workgroup shape (magi_attn_args.q_tile_rows; 0 = the library's choice, which is 256 rows on inputs
+    this small): 256 = 4 waves, 512 = 8 waves of 64 query rows."""
+    q, k, v, bound = _inputs(dn * L, (sp + dn) * L, Hq, Hkv, seed=4321 + L)
+    assert bound <= M.MAGI_SCORE_BOUND_MAX
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    ref = O.range_attention(q, k, v, qr, kr, softmax_scale=LN2)  # q carries softmax_scale * log2(e)
+    lse_ref = O.range_attention_lse(q, k, v, qr, kr, softmax_scale=LN2)
+    tq, tk = _ranges(dev, qr, kr)
+    out, lse = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, int(kr.max() - kr.min()),
+                                 q_prescaled=True, score_bound=bound, q_tile_rows=rows)
+    _cmp(out, ref, f"L={L}")
+    assert (lse.cpu() - lse_ref).abs().max() < 5e-3
+    # against the online-softmax kernel on the same inputs: the same softmax up to the rounding of p to bf16
+    # (relative to the row maximum there, to 2^score here)
+    base, _ = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, q_prescaled=True)
+    assert (out.float() - base.float()).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("gain", [0.25, 1.9])
+def test_bounded_extreme_score_ranges(dev, gain):
+    """Scores near the upper end of the allowed bound (2^+-59 next to each other in one row sum) and tiny ones."""
+    L, dn, sp, Hq, Hkv = 160, 2, 1, 4, 2
+    q, k, v, bound = _inputs(dn * L, (sp + dn) * L, Hq, Hkv, seed=99, gain=gain)
+    assert bound <= M.MAGI_SCORE_BOUND_MAX
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    ref = O.range_attention(q, k, v, qr, kr, softmax_scale=LN2)
+    tq, tk = _ranges(dev, qr, kr)
+    out, _ = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, q_prescaled=True, score_bound=bound)
+    assert torch.isfinite(out).all()
+    _cmp(out, ref, f"gain={gain}")
+
+
+def test_bound_above_the_limit_falls_back_to_the_running_maximum(dev):
+    L, Hq, Hkv = 96, 2, 1
+    q, k, v, _ = _inputs(L, L, Hq, Hkv, seed=5, gain=4.0)  # |q . k| up to ~260: 2^score overflows fp32
+    qr = kr = np.array([[0, L]])
+    tq, tk = _ranges(dev, qr, kr)
+    base, _ = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, q_prescaled=True)
+    out, _ = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, q_prescaled=True, score_bound=300.0)
+    assert torch.equal(out, base)
+
+
+def test_bounded_varlen_segments_with_empty_and_ragged_keys(dev):
+    """cu_seqlens ranges as the T5 cross attention uses them: key segments of 0, 1, 31, 32, 33, 64, 65, 800 tokens."""
+    Lq, Hq, Hkv = 300, 6, 2
+    lens = [0, 1, 31, 32, 33, 64, 65, 800]
+    cu_q = np.arange(0, (len(lens) + 1) * Lq, Lq)
+    cu_k = np.concatenate([[0], np.cumsum(lens)])
+    q, k, v, bound = _inputs(int(cu_q[-1]), int(cu_k[-1]), Hq, Hkv, seed=17)
+    ref = O.varlen_cross_attention(q, k, v, torch.tensor(cu_q), torch.tensor(cu_k), softmax_scale=LN2)
+    tq, tk = _ranges(dev, cu_q, cu_k)
+    out, lse = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, Lq, 800, ranges_mode=M.MAGI_RANGES_CU,
+                                 q_prescaled=True, score_bound=bound)
+    assert torch.all(out[:Lq] == 0) and torch.all(torch.isinf(lse[:, :Lq]))
+    _cmp(out, ref)
+
+
+def test_bounded_cache_views_two_segments_and_grouped_output(dev):
+    """K / V read in place from an interleaved cache, the key axis split into [cache prefix | side buffer] at
+    tile-unfriendly places, and the output written in the two-level head layout: all bit-identical to the plain call."""
+    L, sp, dn, Hq, Hkv, D = 90, 2, 3, 8, 2, 128
+    q, k, v, bound = _inputs(dn * L, (sp + dn) * L, Hq, Hkv, seed=8)
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    tq, tk = _ranges(dev, qr, kr)
+    kw = dict(q_prescaled=True, score_bound=bound)
+    base = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, **kw)[0]
+    _cmp(base, O.range_attention(q, k, v, qr, kr, softmax_scale=LN2))
+    cache = torch.cat([k, v], -1).to(dev)
+    out = M.range_attention(q.to(dev), cache[..., :D], cache[..., D:], tq, tk, L, **kw)[0]
+    assert torch.equal(out, base)
+    for split in (0, sp * L, sp * L + 37, (sp + dn) * L):
+        big = torch.full((split + 5, Hkv, 2 * D), float("nan"), dtype=torch.bfloat16, device=dev)
+        big[:split] = cache[:split]
+        tail = cache[split:].clone()
+        o2 = M.range_attention(q.to(dev), big[:split, :, :D], big[:split, :, D:], tq, tk, L, k2=tail[..., :D],
+                               v2=tail[..., D:], k_split=split, **kw)[0]
+        assert torch.equal(o2, base), f"split={split}"
+    grouped = torch.zeros(dn * L, 4, Hq // 4, D, dtype=torch.bfloat16, device=dev)[:, :, :, :]
+    M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, out=grouped, return_lse=False, **kw)
+    assert torch.equal(grouped.view(dn * L, Hq, D), base)
+
+
+def test_score_bound_argument_checks(dev):
+    q = torch.zeros(4, 1, 128, dtype=torch.bfloat16, device=dev)
+    r = torch.tensor([[0, 4]], dtype=torch.int32, device=dev)
+    with pytest.raises(M.MagiError):  # the bound is in the units of a pre-scaled q
+        M.range_attention(q, q, q, r, r, 4, score_bound=8.0)
+    with pytest.raises(M.MagiError):
+        M.range_attention(q, q, q, r, r, 4, q_prescaled=True, score_bound=-1.0)
+    with pytest.raises(M.MagiError):  # 384-row workgroups belong to the online-softmax kernel
+        M.range_attention(q, q, q, r, r, 4, q_prescaled=True, score_bound=8.0, q_tile_rows=384)
+    with pytest.raises(M.MagiError):
+        M.range_attention(q, q, q, r, r, 4, q_tile_rows=512)

@@ -141,7 +141,9 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.ranges_mode = p->ranges_mode;
   // Kernel choice for bf16.
   //  * Scores with a promised bound (score_bound): the kernel without a running maximum that holds 64 query rows per
-  //    wavefront (every K / V fragment read from LDS feeds two MFMAs); 256-row workgroups (4 waves, two per CU).
+  //    wavefront (every K / V fragment read from LDS feeds two MFMAs); 256-row workgroups (4 waves, two per CU:
+  //    the two waves of a SIMD belong to different workgroups and drift out of step, so one computes scores while
+  //    the other is in its softmax).
   //  * Otherwise 32 rows per wavefront with the online softmax: 384-row workgroups (12 waves, one workgroup per CU,
   //    every K / V tile fetched once for three times as many rows and one barrier per tile) pay on grids of many
   //    rounds with long key ranges (measured: +3 % at 43 rounds, +1 % at 9.4, -3 % at 5.3); small grids and short
@@ -154,7 +156,7 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     const double wg384 = (double)p->Hq * p->n_ranges * ((p->max_seqlen_q + 383) / 384);
     const bool long_keys = p->max_seqlen_k == 0 || p->max_seqlen_k >= 4096;  // (0 = not stated)
     if (bounded)
-      a.block_m = (wg384 >= 9.0 * compute_units() && long_keys) ? 512 : 256;
+      a.block_m = 256;  // (512-row workgroups fetch half the tiles and measure 1 % slower: their two waves per SIMD march in step)
     else if (wg384 >= 9.0 * compute_units() && long_keys)
       a.block_m = 384;
     if (p->q_tile_rows != 0) {

@@ -531,7 +531,11 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 #pragma unroll
       for (int v = (t == 0 ? 3 : 0); v < 16; v += 2) mx = max3(mx, s_acc[t][v], s_acc[t][v + 1 < 16 ? v + 1 : v]);
     mx = half_swap_max(mx);
-    float psum = 0.f;  // row sum of the probabilities as rounded to bf16, i.e. of what the PV product uses
+    // Row sum of the probabilities in fp32, by plain additions.  (v_dot2c_f32_bf16 against (1, 1) would add a packed
+    // pair in one instruction, but dot instructions do not execute beside an MFMA: each one holds the matrix pipe up
+    // for about 16 cycles, measured, where exp2 / convert / add / fma run under it for free.  Rounding to bf16 is
+    // unbiased, so the sum of the unrounded values is as good a denominator.)
+    float psum = 0.f, psum2 = 0.f;
     if constexpr (PRESC) {
       // s_acc holds exponent - m_run: a positive value is a new row maximum (rare after the first tiles)
       const bool raise = first || mx > 0.f;
@@ -559,6 +563,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
         for (int e = 0; e < 8; e += 2) {
           f32x16& sv = s_acc[s >> 1];
           const int v0 = 8 * (s & 1) + e;
+          // (this instantiation has no register left for the two exponentials to outlive their packing: it keeps
+          // the one-instruction pair sum on the packed values)
           const unsigned pk = pack_bf16x2(__builtin_amdgcn_exp2f(sv[v0]), __builtin_amdgcn_exp2f(sv[v0 + 1]));
           psum = pair_sum(pk, psum);
           sv[8 * (s & 1) + (e >> 1)] = __builtin_bit_cast(float, pk);
@@ -586,11 +592,11 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
         const int v0 = 8 * (s & 1) + e;
         const float p0 = __builtin_amdgcn_exp2f(sv[v0] * c - mc);
         const float p1 = __builtin_amdgcn_exp2f(sv[v0 + 1] * c - mc);
-        const unsigned pk = pack_bf16x2(p0, p1);
-        psum = pair_sum(pk, psum);
-        sv[8 * (s & 1) + (e >> 1)] = __builtin_bit_cast(float, pk);
+        psum += p0;
+        psum2 += p1;
+        sv[8 * (s & 1) + (e >> 1)] = __builtin_bit_cast(float, pack_bf16x2(p0, p1));
       }
-    l_run = l_run * alpha + psum;
+    l_run = l_run * alpha + (psum + psum2);
     if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // some row of this wave saw a new maximum
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb)

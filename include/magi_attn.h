@@ -100,6 +100,14 @@ const char* magi_last_error(void);
  *                        times the pre-scale factor.  Larger bounds fall back to the running maximum.  A promise
  *                        that does not hold gives inf / nan or wrong rows, not a fault.  No counterpart in the
  *                        reference.
+ * q_norm_gamma, q_norm_beta, q_norm_eps, q_norm_kind
+ *                        optional (gamma NULL = off): q holds the RAW query projection and the kernel applies the
+ *                        per-(token, head) norm of magi_head_norm (gamma stored zero-centred, beta may be NULL,
+ *                        kind MAGI_NORM_LAYERNORM_1P or MAGI_NORM_RMSNORM_1P) in fp32 while it loads q, multiplies
+ *                        by softmax_scale * log2(e) and rounds to bf16 once.  Stands in for q_layernorm_xattn in
+ *                        get_xqkv (dit_module.py:1008) without the normalised copy of q ever reaching memory.
+ *                        Needs bf16 inputs and a score_bound (stated for the normalised, scaled q); do not set
+ *                        MAGI_ATTN_Q_PRESCALED (the raw q is not scaled).
  * q_tile_rows            0 = the library picks the workgroup shape from the size of the launch.  Otherwise the
  *                        number of query rows per workgroup to use: 128 or 384 (bf16), 256 or 512 (bf16 with a
  *                        score_bound in force), 128 (fp8); anything else is MAGI_EINVAL.  Results do not depend on
@@ -136,6 +144,10 @@ typedef struct magi_attn_args {
   int64_t o_stride_g;
   float score_bound;
   int32_t q_tile_rows;
+  const float* q_norm_gamma;
+  const float* q_norm_beta;
+  float q_norm_eps;
+  int32_t q_norm_kind;
 } magi_attn_args;
 
 int magi_attn_fwd(const magi_attn_args* args, void* stream);

@@ -94,8 +94,21 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   if (p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_FP8_POW2_PRESCALED))
     return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_FP8_POW2_PRESCALED is an fp8 flag");
   if (!(p->score_bound >= 0.f)) return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound must be >= 0");
-  if (p->score_bound > 0.f && !(p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)))
-    return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound needs bf16 inputs with MAGI_ATTN_Q_PRESCALED");
+  const bool q_norm = p->q_norm_gamma != nullptr;
+  if (q_norm) {
+    if (p->dtype != MAGI_DTYPE_BF16 || (p->flags & MAGI_ATTN_Q_PRESCALED))
+      return fail(MAGI_EINVAL, "magi_attn_fwd: q_norm takes raw bf16 q (no MAGI_ATTN_Q_PRESCALED)");
+    if (!(p->score_bound > 0.f && p->score_bound <= MAGI_SCORE_BOUND_MAX))
+      return fail(MAGI_ENOSYS, "magi_attn_fwd: q_norm is implemented for bounded scores (0 < score_bound <= %g)",
+                  (double)MAGI_SCORE_BOUND_MAX);
+    if (p->q_norm_kind != MAGI_NORM_LAYERNORM_1P && p->q_norm_kind != MAGI_NORM_RMSNORM_1P)
+      return fail(MAGI_EINVAL, "magi_attn_fwd: q_norm_kind %d", p->q_norm_kind);
+    if (!(p->q_norm_eps >= 0.f)) return fail(MAGI_EINVAL, "magi_attn_fwd: q_norm_eps");
+    if (!aligned16(p->q_norm_gamma) || !aligned16(p->q_norm_beta))
+      return fail(MAGI_EINVAL, "magi_attn_fwd: q_norm parameters must be 16-byte aligned");
+  }
+  if (p->score_bound > 0.f && !q_norm && !(p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)))
+    return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound needs bf16 inputs with MAGI_ATTN_Q_PRESCALED (or q_norm)");
   if (p->out_group_heads < 0 || (p->out_group_heads > 0 && (p->Hq % p->out_group_heads || p->o_stride_g % 8)))
     return fail(MAGI_EINVAL, "magi_attn_fwd: out_group_heads must divide Hq and o_stride_g keep rows 16-byte aligned");
   int k_split = p->total_k;
@@ -121,6 +134,10 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.lse = p->lse;
   a.q_ranges = p->q_ranges;
   a.k_ranges = p->k_ranges;
+  a.q_norm_gamma = p->q_norm_gamma;
+  a.q_norm_beta = p->q_norm_beta;
+  a.q_norm_eps = p->q_norm_eps;
+  a.q_norm_kind = p->q_norm_kind;
   a.q_scale = p->q_scale;
   a.k_scale = p->k_scale;
   a.v_scale = p->v_scale;
@@ -161,6 +178,7 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
       a.block_m = 384;
     if (p->q_tile_rows != 0) {
       const int r = p->q_tile_rows;
+      if (q_norm && r != 256) return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (with q_norm: 256)", r);
       if (bounded ? (r != 256 && r != 512) : (r != 128 && r != 384))
         return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (bf16: 128 or 384; with a score bound: 256 or 512)", r);
       a.block_m = r;
@@ -184,6 +202,7 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 1.0f / std::sqrt((float)p->D);
   a.scale_log2 = scale * 1.4426950408889634f;
   if (p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)) a.scale_log2 = 1.f;  // q . k is the exp2 exponent
+  // (with q_norm the kernel multiplies the normalised q by scale_log2 itself, after which the same holds)
 
   hipError_t e;
   if (p->dtype != MAGI_DTYPE_BF16)

@@ -51,7 +51,7 @@ __device__ __forceinline__ float keep_lanes(float p, unsigned long long m) {
   return r;
 }
 
-template <int NW, int OCC, bool BOUNDED, int VPRE, int RD, bool PIPE = false>
+template <int NW, int OCC, bool BOUNDED, int VPRE, int RD, bool PIPE = false, bool QNORM = false>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const AttnKernArgs a) {
   constexpr int BM = 64 * NW;
   constexpr int LW = 4;                 // waves that load tiles (the last LW of the workgroup)
@@ -89,6 +89,56 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const A
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) qf[b][kk] = *(const bf16x8*)(qp + kk * 32);
   }
+  if constexpr (QNORM) {
+    // q holds the raw projection: per-(token, head) norm over the 128 features in fp32, times the softmax scale,
+    // one rounding to bf16 (the cross-attention query norm, folded into this kernel's Q load).  A row's features
+    // are spread over the lane pair (i, 0), (i, 1): 64 each, feature 16 kk + 8 g + e in fragment kk, element e.
+    const float inv_d = 1.f / 128.f;
+    float mean[2], rstd[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      float sum = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += (float)qf[b][kk][e];
+      sum += __shfl_xor(sum, 32);
+      mean[b] = a.q_norm_kind == 0 ? sum * inv_d : 0.f;  // (RMS form: no centring)
+      float sq = 0.f;
+#pragma unroll
+      for (int kk = 0; kk < 8; ++kk)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float d = (float)qf[b][kk][e] - mean[b];
+          sq += d * d;
+        }
+      sq += __shfl_xor(sq, 32);
+      rstd[b] = __builtin_amdgcn_rsqf(sq * inv_d + a.q_norm_eps) * a.scale_log2;
+    }
+    // (one fragment index at a time, so that the parameters of one fragment are all that is in registers)
+#pragma unroll
+    for (int kk = 0; kk < 8; ++kk) {
+      __builtin_amdgcn_sched_barrier(0);
+      const f32x4* gp = (const f32x4*)(a.q_norm_gamma + 16 * kk + 8 * g);
+      const f32x4 g0 = gp[0], g1 = gp[1];
+      f32x4 b0 = {0.f, 0.f, 0.f, 0.f}, b1 = b0;
+      if (a.q_norm_beta) {
+        const f32x4* bp = (const f32x4*)(a.q_norm_beta + 16 * kk + 8 * g);
+        b0 = bp[0];
+        b1 = bp[1];
+      }
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+          const float gm = (e < 4 ? g0[e & 3] : g1[e & 3]) + 1.f;
+          const float bt = (e < 4 ? b0[e & 3] : b1[e & 3]) * a.scale_log2;
+          qf[b][kk][e] = (__bf16)(((float)qf[b][kk][e] - mean[b]) * rstd[b] * gm + bt);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+
   // ---- K/V tile loader: loading wave wl fills rows 4*(wl + LW*j) .. +3; lane l sits at row +(l >> 4), slot l & 15 ----
   const int wl = w - (NW - LW);
   const long ks_t = a.ks_t, vs_t = a.vs_t;
@@ -551,7 +601,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const A
 
 hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  const bool bounded = (a.flags & ATTN_BOUNDED) != 0;
+  [[maybe_unused]] const bool bounded = (a.flags & ATTN_BOUNDED) != 0;
+#ifdef MAGI_TUNING  // (tuning builds can also run the 64-row kernels with the running maximum: slower, it spills)
 #define MAGI_W64_LAUNCH(NW, OCC, VPRE, RD)                                                                              \
   do {                                                                                                                   \
     if (bounded)                                                                                                         \
@@ -559,6 +610,10 @@ hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream) {
     else                                                                                                                 \
       hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<NW, OCC, false, VPRE, RD>), dim3(grid), dim3(64 * NW), 0, stream, a); \
   } while (0)
+#else
+#define MAGI_W64_LAUNCH(NW, OCC, VPRE, RD) \
+  hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<NW, OCC, true, VPRE, RD>), dim3(grid), dim3(64 * NW), 0, stream, a)
+#endif
 #ifdef MAGI_TUNING
   if (a.variant == 20)  // software-pipelined loop, one wave per SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 1, true, 0, 4, true>), dim3(grid), dim3(256), 0, stream, a);
@@ -568,7 +623,9 @@ hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream) {
     MAGI_W64_LAUNCH(4, 2, 0, 2);
   else
 #endif
-  if (a.block_m == 512)  // 8 waves, one workgroup per CU: every K / V tile fetched once for 512 rows
+  if (a.q_norm_gamma)  // raw q, normalised while it is loaded (cross attention)
+    hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 2, true, 0, 4, false, true>), dim3(grid), dim3(256), 0, stream, a);
+  else if (a.block_m == 512)  // 8 waves, one workgroup per CU: every K / V tile fetched once for 512 rows
     MAGI_W64_LAUNCH(8, 1, 0, 4);
   else  // 4 waves, two workgroups per CU
     MAGI_W64_LAUNCH(4, 2, 0, 4);

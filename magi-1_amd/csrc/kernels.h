@@ -19,6 +19,8 @@ struct AttnKernArgs {
   const float* q_scale;
   const float* k_scale;
   const float* v_scale;
+  const float* q_norm_gamma;  // non-null: q is raw, normalise each (token, head) row while loading it
+  const float* q_norm_beta;
   long qs_t, qs_h, ks_t, ks_h, vs_t, vs_h, os_t, os_h;
   long os_g;     // byte stride between output head groups (out_group > 0)
   int out_group; // heads per output group, 0 = heads addressed by os_h alone
@@ -31,6 +33,8 @@ struct AttnKernArgs {
   int flags;  // MAGI_ATTN_* bits of the public header, plus ATTN_BOUNDED
   unsigned total_wgs, per_xcd;
   float scale_log2;  // softmax_scale * log2(e)
+  float q_norm_eps;
+  int q_norm_kind;  // MAGI_NORM_LAYERNORM_1P / MAGI_NORM_RMSNORM_1P
 };
 
 

@@ -46,6 +46,7 @@ class AttnArgs(C.Structure):
         ("softmax_scale", C.c_float), ("flags", C.c_int32),
         ("out_group_heads", C.c_int32), ("o_stride_g", C.c_int64), ("score_bound", C.c_float),
         ("q_tile_rows", C.c_int32),
+        ("q_norm_gamma", C.c_void_p), ("q_norm_beta", C.c_void_p), ("q_norm_eps", C.c_float), ("q_norm_kind", C.c_int32),
     ]
 
 

@@ -69,6 +69,7 @@ def range_attention(
     q_prescaled: bool = False,
     score_bound: float = 0.0,
     q_tile_rows: int = 0,
+    q_norm: Optional[tuple] = None,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = True,
     zero_init: bool = True,
@@ -83,6 +84,8 @@ def range_attention(
 
     score_bound (with q_prescaled): promise that |q . k| <= score_bound for every pair; see magi_attn_args.score_bound.
     q_tile_rows: force a workgroup shape (0 = the library's choice); see magi_attn_args.q_tile_rows.
+    q_norm: (gamma, beta or None, eps[, norm_kind]): q is the raw projection, normalised per (token, head) row inside
+    the kernel (fp32, zero-centred gamma) and scaled by softmax_scale * log2(e); needs score_bound.
     """
     _check_thd(q, "q")
     _check_thd(k, "k")
@@ -141,6 +144,14 @@ def range_attention(
     a.flags = (L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0) | (L.MAGI_ATTN_Q_PRESCALED if q_prescaled else 0)
     a.score_bound = float(score_bound)
     a.q_tile_rows = int(q_tile_rows)
+    keep = None
+    if q_norm is not None:
+        g_ = q_norm[0].to(torch.float32).contiguous()
+        b_ = None if q_norm[1] is None else q_norm[1].to(torch.float32).contiguous()
+        keep = (g_, b_)  # (alive until the launch is enqueued)
+        a.q_norm_gamma, a.q_norm_beta = _ptr(g_), _ptr(b_)
+        a.q_norm_eps = float(q_norm[2])
+        a.q_norm_kind = int(q_norm[3]) if len(q_norm) > 3 else L.MAGI_NORM_LAYERNORM_1P
     with torch.cuda.device(q.device):
         L.check(L.lib().magi_attn_fwd(C.byref(a), _stream()))
     return out, lse

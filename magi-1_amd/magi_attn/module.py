@@ -67,6 +67,13 @@ class FusedLayerNorm(torch.nn.Module):
         g = ((w + 1).float() - 1.0) if self.zero_centered_gamma else (w.float() - 1.0)
         return g, self.bias.detach().float()
 
+    def output_norm_bound(self) -> float:
+        """Upper bound of the Euclidean norm of any output row: the normalised row has norm <= sqrt(n) (exactly
+        sqrt(n) up to eps), so |y| <= sqrt(n) max|gamma + 1| + |beta|.  One host read of the parameters."""
+        g, b = self.gamma_beta_fp32()
+        n = g.numel()
+        return float(math.sqrt(n) * (g + 1.0).abs().max().item() + b.norm().item())
+
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         g, b = self.gamma_beta_fp32()
         shape = x.shape
@@ -183,6 +190,22 @@ class FullyParallelAttention(torch.nn.Module):
         self.k_layernorm = mk(torch.float32)
         self.q_layernorm_xattn = mk(params_dtype)
         self.k_layernorm_xattn = mk(params_dtype)
+
+    # ------------------------------------------------------------------ score bounds
+    def score_bounds(self) -> Tuple[float, float]:
+        """(self attention, cross attention) upper bounds of |q . k| in exp2-exponent units (q carrying
+        softmax_scale * log2(e)), from the norm parameters: QK-normed rows have a known length, and the rotary
+        embedding preserves it.  Cauchy-Schwarz, plus 1 % for the roundings to bf16.  Within
+        MAGI_SCORE_BOUND_MAX the attention kernels then need no running maximum (magi_attn_args.score_bound);
+        larger values make them fall back to it.  Computed once per set of parameter values (it reads them on the
+        host) and cached until a parameter is modified or replaced."""
+        lns = (self.q_layernorm, self.k_layernorm, self.q_layernorm_xattn, self.k_layernorm_xattn)
+        key = tuple((id(t), t._version) for ln in lns for t in (ln.weight, ln.bias))
+        if getattr(self, "_bounds_key", None) != key:
+            nq, nk, nqx, nkx = (ln.output_norm_bound() for ln in lns)
+            self._bounds = (1.01 * self._q_premul * nq * nk, 1.01 * self._q_premul * nqx * nkx)
+            self._bounds_key = key
+        return self._bounds
 
     # ------------------------------------------------------------------ cache
     def _allocate_key_and_value_memory(self, sequence_length: int, batch_size: int, dtype) -> torch.Tensor:
@@ -302,9 +325,10 @@ class FullyParallelAttention(torch.nn.Module):
         return q, kv[..., :D].contiguous(), kv[..., D:].contiguous()
 
     def _fused_qkv(self, mixed_qqkv, cos_emb, sin_emb, want_q=True, kv_out=None, n_cache_rows=None, kv_tail=None,
-                   raw=None, q_premul=1.0):
+                   raw=None, q_premul=1.0, rope=None):
         """raw: (q_raw, k_raw, v_raw) already projected (views of forward_qkvx's result), else projected here.
-        q_premul: factor folded into q ahead of its rounding to bf16 (see qk_prologue)."""
+        q_premul: factor folded into q ahead of its rounding to bf16 (see qk_prologue).
+        rope: the [S, 2*R2] sin | cos table when the caller has it in one piece (else built from the two halves)."""
         sq, b = mixed_qqkv.shape[0], mixed_qqkv.shape[1]
         S = sq * b
         Hq, Hkv = self.num_attention_heads, self.num_query_groups_per_partition
@@ -317,7 +341,8 @@ class FullyParallelAttention(torch.nn.Module):
                 q_raw = self.linear_qkv.forward_q(mixed_qqkv).reshape(S, -1)
             else:
                 q_raw = k_raw[:, :0]
-        rope = torch.cat([sin_emb, cos_emb], dim=-1).float().contiguous()
+        if rope is None:
+            rope = torch.cat([sin_emb, cos_emb], dim=-1).float().contiguous()
         gq, bq = self.q_layernorm.gamma_beta_fp32()
         gk, bk = self.k_layernorm.gamma_beta_fp32()
         q, kv, tail = qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, Hq=Hq if want_q else 0, Hkv=Hkv,
@@ -363,26 +388,36 @@ class FullyParallelAttention(torch.nn.Module):
 
     def core_attention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, bs: int,
                        meta_args: ModelMetaArgs, out: Optional[torch.Tensor] = None,
-                       q_prescaled: bool = False) -> torch.Tensor:
+                       q_prescaled: bool = False, score_bound: float = 0.0) -> torch.Tensor:
         """query [(sq b), Hq, D], key / value [(sk b), Hkv, D] -> [(sq b), Hq, D]; dit_module.py:1023-1066.
         bs > 1 only occurs with one range per batch row (asserted there too).  `out` (bs == 1 only) is a
         destination view, possibly in the grouped layout of range_attention.  q_prescaled: query carries
-        softmax_scale * log2(e) (see range_attention)."""
+        softmax_scale * log2(e); score_bound: see range_attention."""
         p = meta_args.core_attn_params
         if bs == 1:
             out, _ = range_attention(query, key, value, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                     out=out, return_lse=False, q_prescaled=q_prescaled)
+                                     out=out, return_lse=False, q_prescaled=q_prescaled, score_bound=score_bound)
             return out
         if meta_args.denoising_range_num > 1:
             raise ValueError("bs > 1 with several denoising ranges is not a layout the pipeline produces")
-        out = torch.zeros_like(query)
-        sq = query.shape[0] // bs
-        one = torch.tensor([[0, sq]], dtype=torch.int32, device=query.device)
-        kone = torch.tensor([[0, key.shape[0] // bs]], dtype=torch.int32, device=query.device)
-        for b in range(bs):  # batch rows are strided views of the (sq b) token axis: no transposes
-            range_attention(query[b::bs], key[b::bs], value[b::bs], one, kone, sq, key.shape[0] // bs,
-                            out=out[b::bs], return_lse=False, q_prescaled=q_prescaled)
-        return out
+        # Batch rows attend to themselves over the whole sequence (dit_module.py:1046-1050): with the token axis
+        # ordered (position, batch) that is ONE range over positions with bs * Hq heads, since head b * Hq + h of
+        # the [(sq), (b Hq), D] view uses kv head (b * Hq + h) / (Hq / Hkv) = b * Hkv + h / (Hq / Hkv).
+        sq, sk = query.shape[0] // bs, key.shape[0] // bs
+        Hq, Hkv, D = query.shape[1], key.shape[1], query.shape[2]
+        if not (query.is_contiguous() and key.stride(0) == Hkv * key.stride(1) and value.stride(0) == Hkv * value.stride(1)):
+            raise ValueError("bs > 1 needs the (position, batch, head) axes of q / k / v evenly strided")
+        dev = query.device
+        ranges = getattr(self, "_one_range", None)
+        if ranges is None or ranges[0] != (sq, sk, dev):
+            ranges = ((sq, sk, dev), torch.tensor([[0, sq]], dtype=torch.int32, device=dev),
+                      torch.tensor([[0, sk]], dtype=torch.int32, device=dev))
+            self._one_range = ranges
+        o, _ = range_attention(query.view(sq, bs * Hq, D), key.as_strided((sk, bs * Hkv, D), (bs * key.stride(0), key.stride(1), 1)),
+                               value.as_strided((sk, bs * Hkv, D), (bs * value.stride(0), value.stride(1), 1)),
+                               ranges[1], ranges[2], sq, sk, return_lse=False, q_prescaled=q_prescaled,
+                               score_bound=score_bound)
+        return o.view(sq * bs, Hq, D)
 
     def cross_attention(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor,
                         cross_attn_params: PackedCrossAttnParams, get_xqkv_func: Callable,
@@ -406,6 +441,29 @@ class FullyParallelAttention(torch.nn.Module):
         out = out.view(b, sq, -1)
         return out.transpose(0, 1).contiguous() if b > 1 else out.view(sq, 1, -1)
 
+    def _cross_attention_fused(self, qx_raw: torch.Tensor, key_value_states: torch.Tensor,
+                               cross_attn_params: PackedCrossAttnParams, out: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        """Batch-1 cross attention on the RAW qx projection [sq, 1, Hq*D]: the attention kernel applies
+        q_layernorm_xattn while it loads q (no normalised copy of q in memory) and, the scores of normed q and k
+        being bounded, runs without a running maximum.  Returns None when that path does not apply (then the
+        caller takes get_xqkv + cross_attention); else the [sq, Hq, D]-shaped result (`out` if given)."""
+        bound = self.score_bounds()[1]
+        if qx_raw.shape[1] != 1 or not (0.0 < bound <= L.MAGI_SCORE_BOUND_MAX):
+            return None
+        D = self.hidden_size_per_attention_head
+        sq = qx_raw.shape[0]
+        q = qx_raw.reshape(sq, -1, D)  # row-strided view of the projection
+        kv = torch.nn.functional.linear(key_value_states, self.linear_kv_xattn.weight)
+        kv = kv.view(key_value_states.shape[0], -1, 2 * D)
+        gk, bk = self.k_layernorm_xattn.gamma_beta_fp32()
+        kx = head_norm(kv[..., :D], gk, bk, self.eps)
+        gq, bq = self.q_layernorm_xattn.gamma_beta_fp32()
+        o, _ = range_attention(q, kx, kv[..., D:], cross_attn_params.cu_seqlens_q, cross_attn_params.cu_seqlens_kv,
+                               cross_attn_params.max_seqlen_q, cross_attn_params.max_seqlen_kv,
+                               ranges_mode=L.MAGI_RANGES_CU, out=out, return_lse=False, zero_init=True,
+                               score_bound=bound, q_norm=(gq, bq, self.eps))
+        return o
+
     # ------------------------------------------------------------------ forward
     def forward(self, hidden_states: torch.Tensor, key_value_states: torch.Tensor,
                 inference_params: Optional[InferenceParams], rotary_pos_emb: torch.Tensor, meta_args: ModelMetaArgs,
@@ -418,6 +476,9 @@ class FullyParallelAttention(torch.nn.Module):
         if rotary_pos_emb is None:
             raise ValueError("FullyParallelAttention needs rotary_pos_emb")
         sin_emb, cos_emb = rotary_pos_emb.tensor_split(2, -1)
+        # the incoming table already is the [sin | cos] layout the prologue takes
+        rope = rotary_pos_emb if (rotary_pos_emb.dtype == torch.float32 and rotary_pos_emb.is_contiguous()) else None
+        bound_core = self.score_bounds()[0]
         bs = hidden_states.shape[1]
         sq = hidden_states.shape[0]
         D = self.hidden_size_per_attention_head
@@ -431,6 +492,8 @@ class FullyParallelAttention(torch.nn.Module):
         fused = None
         core_dst = cross_dst = None
         if proj_layout and bs == 1 and Hq % PROJ_GROUPS == 0:
+            # (rows that no q range / cu_seqlens segment covers are left as allocated: the pipeline's ranges cover
+            # every row, dit_model.py:220-222, 246)
             fused = torch.empty(sq, 1, 2 * Hq * D, dtype=hidden_states.dtype, device=hidden_states.device)
             grouped = fused.view(sq, PROJ_GROUPS, 2, Hq // PROJ_GROUPS, D)
             core_dst, cross_dst = grouped[:, :, 0], grouped[:, :, 1]
@@ -440,11 +503,12 @@ class FullyParallelAttention(torch.nn.Module):
         if self.attention_dtype == "fp8":
             if bs != 1 or (use_cache and inference_params.max_batch_size != 1):
                 raise ValueError("the fp8 self-attention runs at batch 1")
-            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw)
+            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw, rope=rope)
             core = self._core_attention_fp8(q, kv, inference_params, meta_args, use_cache, core_dst)
         elif not use_cache:
-            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw, q_premul=self._q_premul)
-            core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst, q_prescaled=True)
+            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw, q_premul=self._q_premul, rope=rope)
+            core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst, q_prescaled=True,
+                                       score_bound=bound_core)
         else:
             if bs != 1 or inference_params.max_batch_size != 1:
                 raise ValueError("the cached path runs at batch 1 (as the reference pipeline does)")
@@ -458,24 +522,34 @@ class FullyParallelAttention(torch.nn.Module):
             if start + n_keep > cache.shape[0]:
                 raise ValueError("KV cache overflow")
             tail = None
-            if n_keep < S:
-                tail = torch.empty(S - n_keep, cache.shape[1], cache.shape[2], dtype=cache.dtype, device=cache.device)
+            if n_keep < S:  # side buffer for the rows that must not be persisted, kept between calls
+                tail = getattr(self, "_kv_tail", None)
+                if (tail is None or tail.shape[0] < S - n_keep or tail.shape[1:] != cache.shape[1:]
+                        or tail.dtype != cache.dtype or tail.device != cache.device):
+                    tail = torch.empty(S - n_keep, cache.shape[1], cache.shape[2], dtype=cache.dtype, device=cache.device)
+                    self._kv_tail = tail
+                tail = tail[:S - n_keep]
             q, _ = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, kv_out=cache[start:], n_cache_rows=n_keep,
-                                   kv_tail=tail, raw=raw, q_premul=self._q_premul)
+                                   kv_tail=tail, raw=raw, q_premul=self._q_premul, rope=rope)
             split = start + n_keep
             kc, vc = cache[:split, :, :D], cache[:split, :, D:]
             if tail is None:
                 core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                          out=core_dst, return_lse=False, q_prescaled=True)
+                                          out=core_dst, return_lse=False, q_prescaled=True, score_bound=bound_core)
             else:
                 core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
                                           k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, out=core_dst,
-                                          return_lse=False, q_prescaled=True)
+                                          return_lse=False, q_prescaled=True, score_bound=bound_core)
         if fused is not None:
-            self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, get_xqkv, out=cross_dst)
+            if self._cross_attention_fused(qx_raw, key_value_states, meta_args.cross_attn_params, cross_dst) is None:
+                self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, get_xqkv, out=cross_dst)
             return fused
         core_attn_out = core.view(sq, bs, -1)
-        xattn_out = self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, get_xqkv)
+        xo = self._cross_attention_fused(qx_raw, key_value_states, meta_args.cross_attn_params, None)
+        if xo is not None:
+            xattn_out = xo.view(sq, 1, -1)
+        else:
+            xattn_out = self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, get_xqkv)
         if proj_layout:
             return attn_linear_proj_input(core_attn_out, xattn_out)
         return core_attn_out, xattn_out

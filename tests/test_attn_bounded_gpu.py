@@ -153,3 +153,46 @@ def test_score_bound_argument_checks(dev):
         M.range_attention(q, q, q, r, r, 4, q_prescaled=True, score_bound=8.0, q_tile_rows=384)
     with pytest.raises(M.MagiError):
         M.range_attention(q, q, q, r, r, 4, q_tile_rows=512)
+
+
+@pytest.mark.parametrize("kind", ["layernorm", "rmsnorm"])
+def test_query_norm_inside_the_kernel(dev, kind):
+    """q_norm: the kernel takes the RAW query projection (a row-strided view, as the fused projection GEMM leaves it),
+    applies the per-head norm while loading it and scales by softmax_scale * log2(e) before the one rounding to
+    bf16.  Oracle: the CPU restatement of the norm (fp32) followed by the range attention; also against the
+    two-launch form (magi_head_norm, then attention on pre-scaled q) to the rounding of q."""
+    Lq, Hq, Hkv, D = 210, 6, 2, 128
+    lens = [0, 57, 800, 64]
+    g = torch.Generator().manual_seed(31)
+    wide = (torch.randn(len(lens) * Lq, Hq * D + 256, generator=g) * 3 + 0.5).bfloat16()
+    q_raw = wide[:, 128:128 + Hq * D].view(-1, Hq, D)  # rows 2 * (Hq * D + 256) bytes apart
+    gamma = torch.randn(D, generator=g) * 0.1
+    beta = torch.randn(D, generator=g) * 0.1
+    k = O.rmsnorm(torch.randn(sum(lens), Hkv, D, generator=g)).bfloat16()
+    v = torch.randn(sum(lens), Hkv, D, generator=g).bfloat16()
+    cu_q = np.arange(0, (len(lens) + 1) * Lq, Lq)
+    cu_k = np.concatenate([[0], np.cumsum(lens)])
+    eps = 1e-6
+    qf = q_raw.float()
+    if kind == "layernorm":
+        qn = torch.nn.functional.layer_norm(qf, (D,), gamma + 1, beta, eps)
+        code = M.MAGI_NORM_LAYERNORM_1P
+    else:
+        qn = qf * torch.rsqrt(qf.pow(2).mean(-1, keepdim=True) + eps) * (gamma + 1) + beta
+        code = M.MAGI_NORM_RMSNORM_1P
+    ref = O.varlen_cross_attention(qn, k, v, torch.tensor(cu_q), torch.tensor(cu_k))  # fp32 q, softmax scale D^-0.5
+    bound = 1.01 * PREMUL * (qn.norm(dim=-1).max() * k.float().norm(dim=-1).max()).item()
+    assert bound <= M.MAGI_SCORE_BOUND_MAX
+    tq, tk = _ranges(dev, cu_q, cu_k)
+    out, lse = M.range_attention(q_raw.to(dev), k.to(dev), v.to(dev), tq, tk, Lq, 800, ranges_mode=M.MAGI_RANGES_CU,
+                                 score_bound=bound, q_norm=(gamma.to(dev), beta.to(dev), eps, code))
+    assert torch.all(out[:Lq] == 0)
+    _cmp(out, ref, kind)
+    if kind == "layernorm":
+        # the two-launch form rounds the normalised q to bf16 BEFORE the scale is applied inside the kernel
+        qh = M.head_norm(q_raw.to(dev), gamma.to(dev), beta.to(dev), eps)
+        two, _ = M.range_attention(qh, k.to(dev), v.to(dev), tq, tk, Lq, 800, ranges_mode=M.MAGI_RANGES_CU)
+        assert (out.float() - two.float()).abs().max().item() <= 2e-2
+    with pytest.raises(M.MagiError):  # needs the bound
+        M.range_attention(q_raw.to(dev), k.to(dev), v.to(dev), tq, tk, Lq, 800, ranges_mode=M.MAGI_RANGES_CU,
+                          q_norm=(gamma.to(dev), beta.to(dev), eps, code))

@@ -35,10 +35,10 @@ Q_PREMUL = 128 ** -0.5 * math.log2(math.e)  # softmax_scale * log2(e) at head_di
 # roundings to bf16, exactly what FullyParallelAttention.score_bounds() derives from the norm parameters.
 SCORE_BOUND = 1.01 * 128 * Q_PREMUL
 # HBM-side bytes per launch on the 720p workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
-# plain copy of known size in the same run (FETCH_SIZE x2.0, WRITE_SIZE x1.0).  NOT measured in this run:
+# plain copy of known size in the same run (both counters read 1.00 x the bytes of the copy).  NOT measured in this run:
 # the figures and the commands that produced them are in profiles/bench_720p_hbm_traffic_pmc.txt
-MEASURED_TRAFFIC = {"720p-24B": {"core": 257.4e9 + 1.07e9, "prologue": 1.449e9 + 1.434e9,
-                                 "layer_norm": 1.0625e9 + 1.0619e9, "cross": 1.07e9 + 1.07e9}}
+MEASURED_TRAFFIC = {"720p-24B": {"core": 70.25e9 + 1.06e9, "prologue": 0.724e9 + 1.4385e9,
+                                 "layer_norm": 0.531e9 + 1.0617e9, "cross": 0.722e9 + 1.379e9}}
 TRAFFIC_SOURCE = "profiles/bench_720p_hbm_traffic_pmc.txt (counter run of this command, not this run)"
 
 
@@ -160,6 +160,9 @@ def prologue_bytes(inp):
     return 2 * (S * Hq * D * 2) + 2 * (S * Hkv * 2 * D * 2) + S * 96 * 4
 
 
+CORE_BOUND = {"value": SCORE_BOUND}  # (--core-kernel online sets it to 0: no promise, online softmax)
+
+
 def run_step(inp, ev=None):
     """One layer-forward of the hot path, as FullyParallelAttention.forward issues it.
     ev: optional dict of event pairs to record around kernels."""
@@ -181,7 +184,7 @@ def run_step(inp, ev=None):
     rec("prologue", 1)
     rec("core", 0)
     M.range_attention(inp["q"], cache[..., :D], cache[..., D:], inp["q_ranges"], inp["k_ranges"], L,
-                      out=inp["out"], return_lse=False, q_prescaled=True, score_bound=SCORE_BOUND)
+                      out=inp["out"], return_lse=False, q_prescaled=True, score_bound=CORE_BOUND["value"])
     rec("core", 1)
     # cross attention: k norm (a few thousand text tokens), then the attention kernel on the RAW qx projection with
     # the q norm applied while q is loaded
@@ -323,6 +326,9 @@ def main():
     ap.add_argument("--workload", default="720p-24B", choices=sorted(WORKLOADS))
     ap.add_argument("--kv-window", default="default", choices=["default", "noise2clean"],
                     help="key ranges: all chunks up to the query's own (default) or the shipped sliding window")
+    ap.add_argument("--core-kernel", default="bounded", choices=["bounded", "online"],
+                    help="core attention: the bounded-score 64-row kernel the layer module uses (default) or, by "
+                         "withholding the score bound, the online-softmax 32-row kernel that generic callers get")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fp8", action="store_true")
     ap.add_argument("--no-accuracy", action="store_true", help="skip the fp32 sampled-row check of the bf16 output")
@@ -337,6 +343,8 @@ def main():
         sys.exit(2)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.core_kernel == "online":
+        CORE_BOUND["value"] = 0.0
     inp = build_inputs(args.workload, dev, kv_window=args.kv_window)
     core_fl, cross_fl = flops_of(inp)
 
@@ -383,7 +391,7 @@ def main():
                                f"+ T5 cross-attention (lens {inp['t5_lens'].tolist()})"
                                + ("" if args.kv_window == "default" else f", sliding-window key ranges {inp['k_ranges_host'].tolist()}"),
                    "core_flops": core_fl, "cross_flops": cross_fl},
-        "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_w64_kernel", "achieved": round(core_tflops, 2),
+        "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_w64_kernel" if args.core_kernel == "bounded" else "attn_fwd_bf16_kernel", "achieved": round(core_tflops, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(core_tflops / PEAK_BF16_TFLOPS, 4),
                      "traffic": traffic.get("core") if args.kv_window == "default" else None,
                      "traffic_source": TRAFFIC_SOURCE, "ms": round(kern_ms["core"], 3),

@@ -295,7 +295,6 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       i32x8 ka[2], va[2];
       f32x16 s_acc[2];
       i32x8 pb;
-      float psum = 0.f;
       ka[0] = read_k(0, 0);
       ka[1] = read_k(0, 1);
       if constexpr (POW2) {
@@ -371,7 +370,6 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           const float p1 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 1]);
           const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2]);
           const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3]);
-          psum += (p0 + p1) + (p2 + p3);
           // v_cvt_pk_fp8_f32 keeps the other half of its destination: start from p0's register (its high half is
           // overwritten by the second conversion) instead of a zeroed one
           int u = __builtin_bit_cast(int, p0);
@@ -379,7 +377,6 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
           pb[n] = u;
         }
-        l_run += psum * unshift;
       } else {
         const float m_new = fmaxf(m_run, mx * c);
         const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
@@ -391,13 +388,12 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           const float p1 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 1] * c - mc);
           const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2] * c - mc);
           const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3] * c - mc);
-          psum += (p0 + p1) + (p2 + p3);
           int u = __builtin_bit_cast(int, p0);  // see the power-of-two branch
           u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
           u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
           pb[n] = u;
         }
-        l_run = l_run * alpha + psum * unshift;
+        l_run *= alpha;
         if (__builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {
 #pragma unroll
           for (int mb = 0; mb < 4; ++mb)
@@ -409,11 +405,25 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         va[0] = read_v(0);
         va[1] = read_v(1);
       }
+      // Row sums on the matrix pipe: ones^T P^T.  One more MFMA per tile (A = 1.0 in every position, written as fp4
+      // so that it takes four registers; it and the result live in the score registers, which are dead by now)
+      // instead of 32 vector additions per lane: this kernel is bound by vector-instruction issue (its 32
+      // exponentials alone take as long as its 8 MFMAs), not by the matrix pipe.  Every row of the product is the
+      // sum over all 64 keys of the probabilities AS ROUNDED to e4m3, i.e. of exactly what the PV product uses, and
+      // both lanes of a query get the full sum.  Issued ahead of the PV MFMAs and read after them.
+      __builtin_amdgcn_sched_barrier(0);
+      i32x8 ones;
+#pragma unroll
+      for (int n = 0; n < 8; ++n) ones[n] = n < 4 ? 0x22222222 : 0;  // fp4 e2m1 1.0 = 0b0010
+      const f32x16 rowsum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, zero16, 4, 0, 0, 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) {  // two V operands in flight, in alternating registers
         o_acc[mb] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(va[mb & 1], pb, o_acc[mb], 0, 0, 0, 0, 0, 0);
         if (mb + 2 < 4) va[mb & 1] = read_v(mb + 2);
       }
+      __builtin_amdgcn_sched_barrier(0);
+      l_run += rowsum[0] * unshift;
     }
     k0 = k1;
     pe = pe1;
@@ -428,7 +438,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   }
 
   if (!wave_on) return;
-  const float l_tot = l_run + __shfl_xor(l_run, 32);
+  const float l_tot = l_run;  // (the row-sum MFMA hands every lane the sum over all keys of its query)
   const float inv = v_max * __builtin_amdgcn_exp2f(-P_SHIFT) / l_tot;
   // A lane holds four consecutive features per (mb, b), its partner in the other half wave the next four: the
   // halves trade the odd-b registers of the lower half for the even-b registers of the upper one, after which

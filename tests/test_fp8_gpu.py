@@ -69,7 +69,9 @@ def test_fp8_attention_parity(dev, L, dn, sp, Hq, Hkv, C):
     assert err <= 4e-2 and cos >= 0.9995, (err, cos)
     lse_ref = O.range_attention_lse(O.dequantize_per_head_chunk(q8.cpu(), qs.cpu(), C),
                                     O.dequantize_per_head_chunk(k8.cpu(), ks.cpu(), C), v, qr, kr)
-    assert (lse.cpu() - lse_ref).abs().max() < 1e-3
+    # the kernel's row sum runs over the probabilities as rounded to e4m3 (what its PV product uses): each is off by
+    # up to 2^-4 relative, the sum of a row's keys by a few 1e-3
+    assert (lse.cpu() - lse_ref).abs().max() < 2e-2
 
 
 @pytest.mark.parametrize("L,dn,sp,Hq,Hkv,C", [(128, 1, 0, 1, 1, 128), (200, 3, 1, 6, 2, 200), (77, 2, 2, 3, 1, 50),
@@ -100,7 +102,7 @@ def test_fp8_pow2_prescaled_mode(dev, L, dn, sp, Hq, Hkv, C):
     err, cos = _per_head(out, O.range_attention(qd, kd, vd, qr, kr, softmax_scale=1.0))
     assert err <= 4e-2 and cos >= 0.9995, (err, cos)
     lse_ref = O.range_attention_lse(qd, kd, vd, qr, kr, softmax_scale=1.0)
-    assert (lse.cpu() - lse_ref).abs().max() < 1e-3
+    assert (lse.cpu() - lse_ref).abs().max() < 2e-2  # (sum of the e4m3-rounded probabilities, see above)
 
 
 @pytest.mark.parametrize("pow2", [False, True])

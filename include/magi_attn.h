@@ -85,7 +85,9 @@ const char* magi_last_error(void);
  * lse                    optional fp32 [Hq, total_q] (NULL to skip)
  * q_ranges, k_ranges     DEVICE int32 arrays, encoding per ranges_mode; clamped to
  *                        [0,total_q] / [0,total_k] in the kernel
- * max_seqlen_q           upper bound of any q range length (host int; sizes the grid)
+ * max_seqlen_q           upper bound of any q range length (host int; sizes the grid: rows of a range beyond
+ *                        max_seqlen_q are NOT computed and stay untouched, without an error, because the ranges
+ *                        live on the device and the call does not synchronise to read them)
  * q_scale,k_scale,v_scale  fp8 only: DEVICE fp32 [n_scale_chunks, H] with the scale of token t
  *                        at [t / scale_chunk_tokens, h]; NULL for bf16
  * softmax_scale          <= 0 selects D^-0.5

@@ -249,14 +249,20 @@ def test_attention_kernels_keep_their_registers():
     flags = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + csrc,
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
              "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage", "-c", "-o", os.devnull]
-    for src, limit in (("attn_fwd_bf16.hip", 0), ("attn_fwd_fp8.hip", 16)):
+    # the 64-row kernel: no scratch at all in the plain instantiations; the one that normalises q while loading it
+    # (template arguments <..., false, true>, mangled ...ELb0ELb1EE) may park values around that prologue, outside the loop
+    for src, limit in (("attn_fwd_bf16.hip", 0), ("attn_fwd_fp8.hip", 16), ("attn_fwd_bf16_w64.hip", 0)):
         r = subprocess.run([hipcc] + flags + [os.path.join(csrc, src)], capture_output=True, text=True, timeout=600)
         assert r.returncode == 0, r.stderr[-2000:]
         names = re.findall(r"Function Name: (\S+)", r.stderr)
         scratch = [int(x) for x in re.findall(r"ScratchSize \[bytes/lane\]: (\d+)", r.stderr)]
         vgprs = [int(x) for x in re.findall(r" VGPRs: (\d+)", r.stderr)]
         assert names and len(names) == len(scratch) == len(vgprs), (len(names), len(scratch), len(vgprs))
+        seen = 0
         for n, sc, vg in zip(names, scratch, vgprs):
             if "attn_fwd" in n:
-                assert sc <= limit, f"{n}: {sc} bytes of scratch per lane"
+                seen += 1
+                lim = 128 if (src == "attn_fwd_bf16_w64.hip" and n.endswith("ELb0ELb1EEEvNS_12AttnKernArgsE")) else limit
+                assert sc <= lim, f"{n}: {sc} bytes of scratch per lane"
                 assert vg <= 256
+        assert seen >= 2

@@ -17,6 +17,11 @@ from oracle import magi_oracle as O
 pytestmark = pytest.mark.gpu
 
 
+def _cosine(a, b):
+    x, y = a.detach().double().cpu().flatten(), b.detach().double().cpu().flatten()
+    return (torch.dot(x, y) / (x.norm() * y.norm()).clamp_min(1e-30)).item()
+
+
 def _ulp_check(a, ref, what=""):
     a, ref = a.cpu(), ref.cpu()
     af, rf = a.float(), ref.float()
@@ -218,6 +223,7 @@ def test_layer_forward_sequence_with_kv_cache(dev):
         for a, b, nm in ((core, core_ref, "core"), (xo, xo_ref, "xattn")):
             err = (a.float().cpu() - b.float()).abs().max().item()
             assert err <= 3e-2, f"step {(sp, dn, update, distill, extra)} {nm}: {err}"
+            assert _cosine(a, b) >= 0.9999, f"step {(sp, dn, update, distill, extra)} {nm}: cosine {_cosine(a, b)}"
         # what the cache holds afterwards must be what the reference's cache would hold
         if has_ip and (extra or sp > 0) and update:
             keep = S - L if distill else S
@@ -259,6 +265,7 @@ def test_layer_batched_cacheless_pass(dev):
                                      torch.tensor([0, L]), torch.tensor([0, int(lens[b])]), has_ip=False)
         assert (core[:, b].float().cpu() - c_ref[:, 0].float()).abs().max() <= 3e-2
         assert (xo[:, b].float().cpu() - x_ref[:, 0].float()).abs().max() <= 3e-2
+        assert _cosine(core[:, b], c_ref[:, 0]) >= 0.9999 and _cosine(xo[:, b], x_ref[:, 0]) >= 0.9999
 
 
 def test_layer_output_in_linear_proj_layout(dev):
@@ -480,3 +487,20 @@ def test_layer_norm_rejects_bad_arguments():
     with pytest.raises(M.MagiError):
         M.layer_norm(torch.zeros(4, 60, dtype=torch.bfloat16, device="cuda"), None, None)
     assert M.layer_norm(x[:0], None, None).shape == (0, 64)
+
+
+def test_rope_table_built_on_the_device_matches_the_oracle(dev):
+    """The table the layer (and the benchmark) builds with device sin / cos for the 720p window (72 latent frames of
+    45 x 80, last 24 kept) against the CPU restatement of the reference's table: fp32 angles up to ~71 rad, where
+    device and host sin / cos implementations may differ in the last bits of their argument reduction."""
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+
+    fr, H, W, dn, sp = 6, 45, 80, 4, 8
+    got = LearnableRotaryEmbeddingCat(128, device=dev).get_embed_for_forward(dn * fr, H, W, sp, dn)
+    want = O.rope_for_forward(dn * fr, H, W, sp, dn)
+    assert got.shape == want.shape == (dn * fr * H * W, 96) and got.dtype == torch.float32
+    assert (got.cpu() - want).abs().max().item() <= 1e-5
+    # and a small odd grid, where the centre row has all-zero spatial angles
+    got = LearnableRotaryEmbeddingCat(128, device=dev).get_embed_for_forward(4, 5, 7, 1, 2)
+    want = O.rope_for_forward(4, 5, 7, 1, 2)
+    assert (got.cpu() - want).abs().max().item() <= 1e-6

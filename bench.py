@@ -235,14 +235,46 @@ def fp8_leg(inp, core_fl, bf16_tflops, steps, ref_rows, ref):
     res = {"kernel": "attn_fwd_fp8_kernel", "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s",
            "accuracy_reference": f"fp32 attention of {ref.shape[0]} sampled query rows x all heads on the bf16 tensors"}
     out8 = torch.empty_like(inp["out"])
+    S, sp, Hq, Hkv = inp["S"], inp["sp"], inp["Hq"], inp["Hkv"]
+    z = inp["zeros"]
     for mode in ("pow2_prescaled", "generic"):
         pow2 = mode == "pow2_prescaled"
         # pow2_prescaled (what the layer module runs): power-of-two scales on the MFMA's block-scale operands,
-        # softmax_scale * log2(e) already in q (inp["q"] carries it from the prologue); generic: any positive scales,
-        # q scaled back so that the kernel's own softmax scale applies
-        q8, qs = M.quantize_fp8(inp["q"], L, premul=1.0 if pow2 else 1.0 / Q_PREMUL, pow2_scales=pow2)
+        # softmax_scale * log2(e) already in q; generic: any positive scales, q scaled back so that the kernel's own
+        # softmax scale applies.  Cached prefix: quantised from the bf16 cache (absmax scales per chunk and head).
         k8, ks = M.quantize_fp8(cache[..., :D], L, pow2_scales=pow2)
         v8, vs = M.quantize_fp8(cache[..., D:], L, pow2_scales=pow2)
+        if pow2:
+            # this step's rows as FullyParallelAttention(attention_dtype="fp8") prepares them, two launches from the
+            # raw projections on: the prologue writes q and k as e4m3 with constant scales from the norm-parameter
+            # bound (gamma = 1, beta = 0 here: no element of a normed row exceeds sqrt(D)), k into the cache rows;
+            # one launch takes v's absmax scales and quantises it
+            q_sc, k_sc = M.pow2_scale_for(Q_PREMUL * math.sqrt(D)), M.pow2_scale_for(math.sqrt(D))
+            q8 = torch.empty(S, Hq, D, dtype=torch.float8_e4m3fn, device=k8.device)
+            qs = torch.full((S // L, Hq), q_sc, device=k8.device)
+            ks[sp:] = k_sc
+
+            def prepare():
+                M.qk_prologue_fp8(inp["q_raw"], inp["k_raw"], inp["rope"], z, z, z, z, Hq=Hq, Hkv=Hkv, q_scale=q_sc,
+                                  k_scale=k_sc, q_premul=Q_PREMUL, q_out=q8, k_out=k8[sp * L:], n_cache_rows=S)
+                M.quantize_fp8_split(inp["v_raw"].view(S, Hkv, D), L, S, v8[sp * L:], vs[sp:], None, None, pow2_scales=True)
+
+            prepare()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                prepare()
+            e1.record()
+            torch.cuda.synchronize()
+            prep_ms = e0.elapsed_time(e1) / steps
+            prep_bytes = S * Hq * D * 3 + S * Hkv * D * 3 * 2 + S * 96 * 4  # raw bf16 in, e4m3 out, rotary table
+            res["operand_preparation"] = {
+                "launches": 2, "kernels": "prologue_kernel<., e4m3> + quantize_groups_kernel", "ms": round(prep_ms, 4),
+                "bytes": prep_bytes, "achieved": round(prep_bytes / (prep_ms * 1e-3) / 1e9, 1), "unit": "GB/s",
+                "frac": round(prep_bytes / (prep_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+        else:
+            q8, qs = M.quantize_fp8(inp["q"], L, premul=1.0 / Q_PREMUL)
         kw = dict(q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L, out=out8, return_lse=False,
                   fp8_pow2_prescaled=pow2)
         M.range_attention(q8, k8, v8, inp["q_ranges"], inp["k_ranges"], L, **kw)

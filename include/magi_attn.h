@@ -150,6 +150,12 @@ typedef struct magi_attn_args {
   const float* q_norm_beta;
   float q_norm_eps;
   int32_t q_norm_kind;
+  /* fp8, optional: scale rows of the side segment k2 / v2 in tables of their own, [chunks of the segment, Hkv],
+   * row 0 = the chunk that starts at k_split (then a multiple of scale_chunk_tokens).  A caller that keeps
+   * k_scale / v_scale next to a persistent cache can so attach rows it must not persist without rewriting the
+   * cache's tables.  NULL (both): k_scale / v_scale are indexed across k_split as one table. */
+  const float* k2_scale;
+  const float* v2_scale;
 } magi_attn_args;
 
 int magi_attn_fwd(const magi_attn_args* args, void* stream);
@@ -173,6 +179,15 @@ int magi_attn_fwd(const magi_attn_args* args, void* stream);
  *         stride kv_stride_t; K goes to [..., 0:D], V to [..., D:2D]
  * kv_tail destination of tokens >= n_cache_rows (same layout, row index t - n_cache_rows); may be
  *         NULL when n_cache_rows == S
+ * out_dtype  MAGI_DTYPE_BF16 (0): as above.  MAGI_DTYPE_FP8_E4M3: the operands of the fp8 attention leave this
+ *         pass directly, with no bf16 copy and no absmax pass:  q_out [S, Hq, D] = sat_e4m3(q * q_premul /
+ *         q_quant_scale), and kv_out / kv_tail are K destinations [*, Hkv, D] e4m3 (token strides in elements)
+ *         = sat_e4m3(k / k_quant_scale).  The two scales are constants of the call (use powers of two: the
+ *         kernel multiplies by the reciprocal, which is then exact): a QK-normed row cannot exceed
+ *         sqrt(D) max|gamma + 1| + |beta| in any element, before or after the rotation, so a scale chosen from
+ *         the norm parameters never saturates, and e4m3 being a floating-point format a conservative scale
+ *         costs no precision.  The attention call takes them as constant q_scale / k_scale tables.  V is not
+ *         touched (v_raw may be NULL): it has no a-priori bound; magi_quantize_fp8_split takes it from v_raw.
  */
 typedef struct magi_prologue_args {
   const void* q_raw;
@@ -194,6 +209,8 @@ typedef struct magi_prologue_args {
   float eps;
   int32_t batch; /* tokens are ordered (position, batch): rope row of token t is t / batch; 0 or 1 = no batch */
   float q_premul;
+  int32_t out_dtype;
+  float q_quant_scale, k_quant_scale;
 } magi_prologue_args;
 
 int magi_qk_prologue(const magi_prologue_args* args, void* stream);
@@ -237,6 +254,30 @@ int magi_apply_rotary(const void* x, const float* cos, const float* sin, void* y
  */
 int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, float* scales, int32_t T,
                       int32_t H, int32_t D, int32_t chunk_tokens, float premul, int32_t pow2_scales, void* stream);
+
+/*
+ * The same quantiser with two destinations, as the KV-cache append has them (dit_module.py:918-929: rows that
+ * are persisted go to the cache, the others only serve this call): tokens below n_rows_first go to y / scales,
+ * the others to y2 / scales2 with row and chunk indices counted from n_rows_first (a multiple of chunk_tokens
+ * unless it equals T; y / scales may be NULL when it is 0, y2 / scales2 when it is T).  Always ONE launch: a
+ * workgroup per (chunk, head) takes the absmax, writes the scale and quantises, with no memory beyond x and the
+ * outputs, so it suits groups the size of a video chunk; magi_quantize_fp8 switches to a multi-launch form for
+ * large groups and gives the same bytes.
+ */
+typedef struct magi_quantize_args {
+  const void* x;
+  int64_t x_stride_t, x_stride_h;
+  int32_t T, H, D, chunk_tokens;
+  float premul;
+  int32_t pow2_scales;
+  void* y;
+  float* scales;
+  int32_t n_rows_first;
+  void* y2;
+  float* scales2;
+} magi_quantize_args;
+
+int magi_quantize_fp8_split(const magi_quantize_args* args, void* stream);
 
 #ifdef __cplusplus
 }

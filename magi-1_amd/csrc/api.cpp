@@ -121,6 +121,10 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   if (p->dtype == MAGI_DTYPE_FP8_E4M3) {
     if (!p->q_scale || !p->k_scale || !p->v_scale || p->scale_chunk_tokens <= 0)
       return fail(MAGI_EINVAL, "magi_attn_fwd: fp8 needs q/k/v scales and scale_chunk_tokens > 0");
+    if ((p->k2_scale != nullptr) != (p->v2_scale != nullptr))
+      return fail(MAGI_EINVAL, "magi_attn_fwd: k2_scale and v2_scale come together");
+    if (p->k2_scale && (!p->k2 || p->k_split % p->scale_chunk_tokens))
+      return fail(MAGI_EINVAL, "magi_attn_fwd: k2_scale / v2_scale need k2 / v2 and k_split on a scale-chunk boundary");
   }
 
   magi::AttnKernArgs a;
@@ -194,6 +198,12 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.Hkv = p->Hkv;
   a.G = p->Hq / p->Hkv;
   a.scale_chunk_tokens = p->scale_chunk_tokens;
+  a.scale_split_chunk = 0x7fffffff;
+  if (p->dtype == MAGI_DTYPE_FP8_E4M3 && p->k2_scale) {
+    a.scale_split_chunk = p->k_split / p->scale_chunk_tokens;
+    a.k2_scale_delta = (p->k2_scale - p->k_scale) - (long)a.scale_split_chunk * p->Hkv;
+    a.v2_scale_delta = (p->v2_scale - p->v_scale) - (long)a.scale_split_chunk * p->Hkv;
+  }
   a.flags = p->flags | (bounded ? magi::ATTN_BOUNDED : 0);
   const double total = (double)p->Hq * p->n_ranges * a.tiles_per_range;
   if (total > 2.0e9) return fail(MAGI_EINVAL, "magi_attn_fwd: grid too large (%.3g workgroups)", total);
@@ -225,7 +235,12 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   if (p->norm_kind < 0 || p->norm_kind > 2) return fail(MAGI_EINVAL, "magi_qk_prologue: norm_kind %d", p->norm_kind);
   if (p->batch < 0) return fail(MAGI_EINVAL, "magi_qk_prologue: negative batch");
   if (p->Hq > 0 && (!p->q_raw || !p->q_out)) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL q_raw/q_out");
-  if (p->Hkv > 0 && (!p->k_raw || !p->v_raw)) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL k_raw/v_raw");
+  const bool out8 = p->out_dtype == MAGI_DTYPE_FP8_E4M3;
+  if (p->out_dtype != MAGI_DTYPE_BF16 && !out8) return fail(MAGI_EINVAL, "magi_qk_prologue: out_dtype %d", p->out_dtype);
+  if (p->Hkv > 0 && (!p->k_raw || (!p->v_raw && !out8))) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL k_raw/v_raw");
+  if (out8 && ((p->Hq > 0 && !(p->q_quant_scale > 0.f && std::isfinite(p->q_quant_scale))) ||
+               (p->Hkv > 0 && !(p->k_quant_scale > 0.f && std::isfinite(p->k_quant_scale)))))
+    return fail(MAGI_EINVAL, "magi_qk_prologue: e4m3 outputs need positive finite q_quant_scale / k_quant_scale");
   if (p->n_cache_rows < 0 || p->n_cache_rows > p->S)
     return fail(MAGI_EINVAL, "magi_qk_prologue: n_cache_rows %d outside [0, S=%d]", p->n_cache_rows, p->S);
   if (p->Hkv > 0 && p->n_cache_rows > 0 && !p->kv_out) return fail(MAGI_EINVAL, "magi_qk_prologue: NULL kv_out");
@@ -238,7 +253,7 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   if (p->q_raw_stride_t % 8 || p->k_raw_stride_t % 8 || p->v_raw_stride_t % 8 || p->kv_stride_t % 8 ||
       p->kv_tail_stride_t % 8)
     return fail(MAGI_EINVAL, "magi_qk_prologue: strides must keep rows 16-byte aligned");
-  if (!aligned16(p->q_raw) || !aligned16(p->k_raw) || !aligned16(p->v_raw) || !aligned16(p->q_out) ||
+  if (!aligned16(p->q_raw) || !aligned16(p->k_raw) || (!out8 && !aligned16(p->v_raw)) || !aligned16(p->q_out) ||
       !aligned16(p->kv_out) || !aligned16(p->kv_tail))
     return fail(MAGI_EINVAL, "magi_qk_prologue: buffers must be 16-byte aligned");
 
@@ -258,8 +273,11 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   a.q_raw_stride_t = p->q_raw_stride_t * 2;
   a.k_raw_stride_t = p->k_raw_stride_t * 2;
   a.v_raw_stride_t = p->v_raw_stride_t * 2;
-  a.kv_stride_t = p->kv_stride_t * 2;
-  a.kv_tail_stride_t = p->kv_tail_stride_t * 2;
+  a.kv_stride_t = p->kv_stride_t * (out8 ? 1 : 2);
+  a.kv_tail_stride_t = p->kv_tail_stride_t * (out8 ? 1 : 2);
+  a.out_fp8 = out8;
+  a.q_inv_scale = out8 && p->Hq > 0 ? 1.f / p->q_quant_scale : 1.f;
+  a.k_inv_scale = out8 && p->Hkv > 0 ? 1.f / p->k_quant_scale : 1.f;
   a.S = p->S;
   a.n_cache_rows = p->n_cache_rows;
   a.Hq = p->Hq;
@@ -322,20 +340,49 @@ int magi_apply_rotary(const void* x, const float* cos, const float* sin, void* y
   return MAGI_OK;
 }
 
-int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, float* scales, int32_t T,
-                      int32_t H, int32_t D, int32_t chunk_tokens, float premul, int32_t pow2_scales, void* stream) {
-  if (D != 128) return fail(MAGI_ENOSYS, "magi_quantize_fp8: head_dim %d not implemented (128 only)", D);
-  if (T < 0 || H < 0 || chunk_tokens <= 0) return fail(MAGI_EINVAL, "magi_quantize_fp8: bad size");
-  if (!(premul == premul) || premul == 0.f) return fail(MAGI_EINVAL, "magi_quantize_fp8: premul must be finite and non-zero");
-  if (T == 0 || H == 0) return MAGI_OK;
-  if (!x || !y || !scales) return fail(MAGI_EINVAL, "magi_quantize_fp8: NULL pointer");
-  if (x_stride_t % 8 || x_stride_h % 8 || !aligned16(x) || !aligned16(y))
+int magi_quantize_fp8_split(const magi_quantize_args* p, void* stream) {
+  if (!p) return fail(MAGI_EINVAL, "magi_quantize_fp8: args is NULL");
+  if (p->D != 128) return fail(MAGI_ENOSYS, "magi_quantize_fp8: head_dim %d not implemented (128 only)", p->D);
+  if (p->T < 0 || p->H < 0 || p->chunk_tokens <= 0) return fail(MAGI_EINVAL, "magi_quantize_fp8: bad size");
+  if (!(p->premul == p->premul) || p->premul == 0.f)
+    return fail(MAGI_EINVAL, "magi_quantize_fp8: premul must be finite and non-zero");
+  if (p->n_rows_first < 0 || p->n_rows_first > p->T)
+    return fail(MAGI_EINVAL, "magi_quantize_fp8: n_rows_first %d outside [0, T=%d]", p->n_rows_first, p->T);
+  if (p->n_rows_first < p->T && p->n_rows_first % p->chunk_tokens)
+    return fail(MAGI_EINVAL, "magi_quantize_fp8: n_rows_first must be a multiple of chunk_tokens");
+  if (p->T == 0 || p->H == 0) return MAGI_OK;
+  if (p->H > 65535) return fail(MAGI_ENOSYS, "magi_quantize_fp8: more than 65535 heads");
+  if (!p->x) return fail(MAGI_EINVAL, "magi_quantize_fp8: NULL pointer");
+  if (p->n_rows_first > 0 && (!p->y || !p->scales)) return fail(MAGI_EINVAL, "magi_quantize_fp8: NULL pointer");
+  if (p->n_rows_first < p->T && (!p->y2 || !p->scales2))
+    return fail(MAGI_EINVAL, "magi_quantize_fp8: y2 / scales2 needed for rows >= n_rows_first");
+  if (p->x_stride_t % 8 || p->x_stride_h % 8 || !aligned16(p->x) || !aligned16(p->y) || !aligned16(p->y2))
     return fail(MAGI_EINVAL, "magi_quantize_fp8: rows must be 16-byte aligned");
-  hipError_t e = magi::launch_quantize_fp8(static_cast<const char*>(x), x_stride_t * 2, x_stride_h * 2,
-                                           static_cast<char*>(y), scales, T, H, chunk_tokens, premul,
-                                           pow2_scales, static_cast<hipStream_t>(stream));
+  hipError_t e = magi::launch_quantize_fp8(static_cast<const char*>(p->x), p->x_stride_t * 2, p->x_stride_h * 2,
+                                           static_cast<char*>(p->y), p->scales, p->T, p->H, p->chunk_tokens, p->premul,
+                                           p->pow2_scales, p->n_rows_first, static_cast<char*>(p->y2), p->scales2,
+                                           static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_quantize_fp8 launch");
   return MAGI_OK;
+}
+
+int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, float* scales, int32_t T,
+                      int32_t H, int32_t D, int32_t chunk_tokens, float premul, int32_t pow2_scales, void* stream) {
+  magi_quantize_args q;
+  std::memset(&q, 0, sizeof(q));
+  q.x = x;
+  q.x_stride_t = x_stride_t;
+  q.x_stride_h = x_stride_h;
+  q.T = T;
+  q.H = H;
+  q.D = D;
+  q.chunk_tokens = chunk_tokens;
+  q.premul = premul;
+  q.pow2_scales = pow2_scales;
+  q.y = y;
+  q.scales = scales;
+  q.n_rows_first = T;
+  return magi_quantize_fp8_split(&q, stream);
 }
 
 }  // extern "C"

@@ -143,7 +143,10 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
 
   // largest V scale of the key range (reference for the relative V scale folded into exp2)
   float v_max = 0.f;
-  for (int cidx = ks / C; cidx <= (ke - 1) / C; ++cidx) v_max = fmaxf(v_max, a.v_scale[(long)cidx * a.Hkv + kvh]);
+  // (the side segment's chunks may have scale tables of their own: reached from the main tables by a constant
+  // element offset from chunk scale_split_chunk on)
+  for (int cidx = ks / C; cidx <= (ke - 1) / C; ++cidx)
+    v_max = fmaxf(v_max, a.v_scale[(long)cidx * a.Hkv + kvh + (cidx < a.scale_split_chunk ? 0 : a.v2_scale_delta)]);
   const float log2_vmax = __builtin_amdgcn_logf(v_max);
 
   // ---- tile loader: wave w fills rows 8*(w + NW*j) .. +7; lane l sits at row +(l >> 3), slot l & 7 ----
@@ -267,8 +270,9 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         auto uni = [](float x) {
           return __builtin_bit_cast(float, __builtin_amdgcn_readfirstlane(__builtin_bit_cast(int, x)));
         };
-        const float k_sc = uni(a.k_scale[(long)chunk * a.Hkv + kvh]);
-        const float v_sc = a.v_scale[(long)chunk * a.Hkv + kvh];
+        const bool side = chunk >= a.scale_split_chunk;
+        const float k_sc = uni(a.k_scale[(long)chunk * a.Hkv + kvh + (side ? a.k2_scale_delta : 0)]);
+        const float v_sc = a.v_scale[(long)chunk * a.Hkv + kvh + (side ? a.v2_scale_delta : 0)];
         if constexpr (!POW2) c = c_q * k_sc;                             // per-lane score scale inside this piece
         shift = uni(P_SHIFT + __builtin_amdgcn_logf(v_sc) - log2_vmax);  // <= 8
         unshift = uni(__builtin_amdgcn_exp2f(-shift));
@@ -503,28 +507,25 @@ __global__ __launch_bounds__(QT) void absmax_kernel(const char* x, long xs_t, lo
   }
 }
 
-__global__ __launch_bounds__(QT) void finalize_scales_kernel(float* scales, int n, float premul, int pow2) {
-  const int i = blockIdx.x * QT + threadIdx.x;
-  if (i >= n) return;
-  float f = fmaxf(scales[i] * fabsf(premul) / 448.f, 1e-12f);
+// absmax of a (chunk, head) group -> its scale
+__device__ __forceinline__ float scale_of_absmax(float amax, float premul, int pow2) {
+  float f = fmaxf(amax * fabsf(premul) / 448.f, 1e-12f);
   if (pow2) {  // round up to a power of two
     unsigned b = __builtin_bit_cast(unsigned, f);
     b = ((b >> 23) + ((b & 0x7fffffu) ? 1u : 0u)) << 23;
     f = __builtin_bit_cast(float, b);
   }
-  scales[i] = f;
+  return f;
 }
 
-// one thread per 8 elements
-__global__ __launch_bounds__(QT) void quantize_kernel(const char* x, long xs_t, long xs_h, char* y, const float* scales,
-                                                      int T, int H, int chunk_tokens, float premul) {
-  const long gid = (long)blockIdx.x * QT + threadIdx.x;
-  const long row = gid >> 4;
-  const int part = (int)(gid & 15);
-  if (row >= (long)T * H) return;
-  const int t = (int)(row / H), h = (int)(row % H);
-  const float sc = scales[(long)(t / chunk_tokens) * H + h];
-  const u32x4 v = *(const u32x4*)(x + (long)t * xs_t + (long)h * xs_h + part * 16);
+__global__ __launch_bounds__(QT) void finalize_scales_kernel(float* scales, int n, float premul, int pow2) {
+  const int i = blockIdx.x * QT + threadIdx.x;
+  if (i >= n) return;
+  scales[i] = scale_of_absmax(scales[i], premul, pow2);
+}
+
+// 16 bytes of bf16 (8 elements) -> 8 bytes of e4m3: y = sat(x * premul / sc)
+__device__ __forceinline__ u32x2 quantize8(const u32x4 v, float premul, float sc) {
   float fv[8];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -541,7 +542,59 @@ __global__ __launch_bounds__(QT) void quantize_kernel(const char* x, long xs_t, 
     u = __builtin_amdgcn_cvt_pk_fp8_f32(fv[4 * j + 2], fv[4 * j + 3], u, true);
     o[j] = (unsigned)u;
   }
-  *(u32x2*)(y + row * 128 + part * 8) = o;
+  return o;
+}
+
+// one thread per 8 elements
+__global__ __launch_bounds__(QT) void quantize_kernel(const char* x, long xs_t, long xs_h, char* y, const float* scales,
+                                                      int T, int H, int chunk_tokens, float premul) {
+  const long gid = (long)blockIdx.x * QT + threadIdx.x;
+  const long row = gid >> 4;
+  const int part = (int)(gid & 15);
+  if (row >= (long)T * H) return;
+  const int t = (int)(row / H), h = (int)(row % H);
+  const float sc = scales[(long)(t / chunk_tokens) * H + h];
+  const u32x4 v = *(const u32x4*)(x + (long)t * xs_t + (long)h * xs_h + part * 16);
+  *(u32x2*)(y + row * 128 + part * 8) = quantize8(v, premul, sc);
+}
+
+// The whole job in one launch, for groups small enough that one workgroup can walk them twice (a video chunk of
+// one head is 0.4 MB at the 720p shape and stays in L2 between the passes): workgroup (h, c) takes the absmax of
+// its (chunk, head) group, reduces it through LDS, writes the scale, and quantises the group with it.  No memory
+// beyond the inputs and outputs.  Groups that start at or after token n_first go to the second destination.
+constexpr int QT1 = 1024;
+__global__ __launch_bounds__(QT1) void quantize_groups_kernel(const char* x, long xs_t, long xs_h, char* y, float* scales,
+                                                              int T, int H, int chunk_tokens, float premul, int pow2,
+                                                              int n_first, char* y2, float* scales2) {
+  __shared__ unsigned s_red[QT1 / 64];
+  const int h = blockIdx.x, c = blockIdx.y;
+  const int t_begin = c * chunk_tokens, t_end = min(T, t_begin + chunk_tokens);
+  const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
+  const char* const xcol = x + (long)h * xs_h + lane16 * 16;
+  unsigned m = 0u;
+  for (int t = t_begin + sub; t < t_end; t += QT1 / 16) {
+    const u32x4 v = *(const u32x4*)(xcol + (long)t * xs_t);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      m = max(m, (v[j] << 16) & 0x7fffffffu);
+      m = max(m, v[j] & 0x7fff0000u);
+    }
+  }
+#pragma unroll
+  for (int o = 32; o >= 1; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o));
+  if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
+  __syncthreads();
+#pragma unroll
+  for (int j = 0; j < QT1 / 64; ++j) m = max(m, s_red[j]);  // non-negative floats order like their bit patterns
+  const float sc = scale_of_absmax(__builtin_bit_cast(float, m), premul, pow2);
+  const bool second = t_begin >= n_first;
+  const int t_off = second ? n_first : 0;
+  if (threadIdx.x == 0) (second ? scales2 : scales)[(long)(c - t_off / chunk_tokens) * H + h] = sc;
+  char* const ycol = (second ? y2 : y) + (long)h * 128 + lane16 * 8;
+  for (int t = t_begin + sub; t < t_end; t += QT1 / 16) {
+    const u32x4 v = *(const u32x4*)(xcol + (long)t * xs_t);
+    *(u32x2*)(ycol + (long)(t - t_off) * H * 128) = quantize8(v, premul, sc);
+  }
 }
 
 }  // namespace
@@ -556,9 +609,20 @@ hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream) {
 }
 
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
-                               int chunk_tokens, float premul, int pow2_scales, hipStream_t stream) {
+                               int chunk_tokens, float premul, int pow2_scales, int n_first, char* y2, float* scales2,
+                               hipStream_t stream) {
   const int n_chunks = (T + chunk_tokens - 1) / chunk_tokens;
   const int n = n_chunks * H;
+  if (n <= 0) return hipSuccess;
+  // One launch when a group fits one workgroup's two passes and there are enough groups to spread over the chip
+  // (or a second destination, which only that kernel serves); both paths give the same bytes.
+  const bool one_launch = n_first < T || (min(chunk_tokens, T) <= 8192 && (n >= 64 || (long)T * H <= 65536));
+  if (one_launch) {
+    if (n_chunks > 65535) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(quantize_groups_kernel, dim3(H, n_chunks), dim3(QT1), 0, stream, x, x_stride_t, x_stride_h, y,
+                       scales, T, H, chunk_tokens, premul, pow2_scales, n_first, y2, scales2);
+    return hipGetLastError();
+  }
   hipLaunchKernelGGL(fill_zero_kernel, dim3((n + QT - 1) / QT), dim3(QT), 0, stream, (unsigned*)scales, n);
   const int rows_per_pass = QT / 16;
   int slices = (min(chunk_tokens, T) + rows_per_pass * 8 - 1) / (rows_per_pass * 8);

@@ -22,6 +22,9 @@ struct AttnKernArgs {
   const float* q_norm_gamma;  // non-null: q is raw, normalise each (token, head) row while loading it
   const float* q_norm_beta;
   long qs_t, qs_h, ks_t, ks_h, vs_t, vs_h, os_t, os_h;
+  // fp8, side segment with scale tables of its own: element offsets that lead from row c of k_scale / v_scale to
+  // row c - scale_split_chunk of those tables (0 without them)
+  long k2_scale_delta, v2_scale_delta;
   long os_g;     // byte stride between output head groups (out_group > 0)
   int out_group; // heads per output group, 0 = heads addressed by os_h alone
   int total_q, total_k, k_split;
@@ -30,6 +33,7 @@ struct AttnKernArgs {
   int variant;  // tuning builds: bf16 kernel instantiation picked by hand (0 = the library's own choice)
   int Hq, Hkv, G;
   int scale_chunk_tokens;
+  int scale_split_chunk;  // first chunk served by the side segment's scale tables (INT_MAX without them)
   int flags;  // MAGI_ATTN_* bits of the public header, plus ATTN_BOUNDED
   unsigned total_wgs, per_xcd;
   float scale_log2;  // softmax_scale * log2(e)
@@ -65,6 +69,8 @@ struct PrologueKernArgs {
   float eps;
   int batch;
   float q_premul;  // factor on q before the bf16 rounding (1 = none)
+  int out_fp8;     // q and k leave as e4m3 (kv_out / kv_tail then hold K rows only, strides in bytes); v untouched
+  float q_inv_scale, k_inv_scale;  // out_fp8: 1 / the constant scale of q (after q_premul) and of k
 };
 hipError_t launch_prologue(const PrologueKernArgs& a, hipStream_t stream);
 
@@ -74,7 +80,10 @@ hipError_t launch_layer_norm(const char* x, long x_stride, const void* w, const 
                              long y_stride, long rows, int cols, float eps, hipStream_t stream);
 hipError_t launch_rotary(const void* x, const float* cos, const float* sin, void* y, int B, int S, int H, int D,
                          int R2, int is_bf16, hipStream_t stream);
+// Rows below n_first go to y / scales, the rest (row index and chunk index counted from n_first, a multiple of
+// chunk_tokens) to y2 / scales2.
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
-                               int chunk_tokens, float premul, int pow2_scales, hipStream_t stream);
+                               int chunk_tokens, float premul, int pow2_scales, int n_first, char* y2, float* scales2,
+                               hipStream_t stream);
 
 }  // namespace magi

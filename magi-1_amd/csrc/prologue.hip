@@ -1,5 +1,7 @@
 // HBM-bound prologue kernels for gfx950: per-head QK norm + partial non-interleaved rotary +
-// bf16 cast + KV-cache write in one pass, plus the norm-only and rotary-only variants.
+// bf16 cast + KV-cache write in one pass, plus the norm-only and rotary-only variants.  With e4m3 outputs the
+// same pass quantises q and k with constant scales (rows of a QK norm have a known bound, so no absmax pass is
+// needed) and leaves v to the chunk quantiser.
 //
 // Layout: 8 lanes serve one (token, head) row of D = 128 elements, 16 elements (two 16-byte
 // vectors) per lane, chosen so that a rotary pair (i, i + R2) lives in ONE lane: lanes
@@ -13,6 +15,7 @@ namespace magi {
 namespace {
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
@@ -38,6 +41,21 @@ __device__ __forceinline__ u32x4 pack8(const float* f) {
 #pragma unroll
   for (int i = 0; i < 4; ++i) v[i] = pack2(f[2 * i], f[2 * i + 1]);
   return v;
+}
+// 8 floats -> 8 saturating OCP e4m3fn bytes (the conversion itself does not saturate: clamp first)
+__device__ __forceinline__ u32x2 pack8_e4m3(const float* f) {
+  u32x2 o;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    float c[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) c[i] = fminf(fmaxf(f[4 * j + i], -448.f), 448.f);
+    int u = 0;
+    u = __builtin_amdgcn_cvt_pk_fp8_f32(c[0], c[1], u, false);
+    u = __builtin_amdgcn_cvt_pk_fp8_f32(c[2], c[3], u, true);
+    o[j] = (unsigned)u;
+  }
+  return o;
 }
 __device__ __forceinline__ float group8_sum(float x) {
   x += __shfl_xor(x, 1);
@@ -77,7 +95,9 @@ __device__ __forceinline__ void norm16(float* x, const float* gam, const float* 
   }
 }
 
-template <int TPB>  // tokens that share a workgroup: 1, 2, 4 or 8
+// TPB: tokens that share a workgroup (1, 2, 4 or 8).  OUT8: q and k leave as e4m3 bytes (q_out [S, Hq, D],
+// K rows [*, Hkv, D] at kv_out / kv_tail), each multiplied by its constant inverse scale; v is not touched.
+template <int TPB, bool OUT8>
 __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArgs a) {
   __shared__ float s_par[4][D];  // gq, bq, gk, bk
   const int tid = threadIdx.x;
@@ -98,7 +118,8 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
   const bool rot_lane = j < nr;
   const int ea = rot_lane ? 8 * j : 2 * a.R2 + 16 * (j - nr);  // first element of vector A
   const int eb = rot_lane ? a.R2 + 8 * j : ea + 8;             // first element of vector B
-  const int U = a.Hq + 2 * a.Hkv;
+  const int U = a.Hq + (OUT8 ? 1 : 2) * a.Hkv;
+  constexpr int ES = OUT8 ? 1 : 2;  // bytes per output element
 
   {
     const int s = blockIdx.x * TPB + team;
@@ -125,12 +146,12 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
       if (u < a.Hq) {
         kind = 0;
         src = a.q_raw + (long)s * a.q_raw_stride_t + (long)u * (D * 2);
-        dst = a.q_out + ((long)s * a.Hq + u) * (D * 2);
+        dst = a.q_out + ((long)s * a.Hq + u) * (D * ES);
       } else if (u < a.Hq + a.Hkv) {
         kind = 1;
         const int hh = u - a.Hq;
         src = a.k_raw + (long)s * a.k_raw_stride_t + (long)hh * (D * 2);
-        dst = kvrow + (long)hh * (2 * D * 2);
+        dst = kvrow + (long)hh * (OUT8 ? D : 2 * D * 2);
       } else {
         kind = 2;
         const int hh = u - a.Hq - a.Hkv;
@@ -160,8 +181,16 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
 #pragma unroll
         for (int i = 0; i < 16; ++i) x[i] *= a.q_premul;
       }
-      *(u32x4*)(dst + ea * 2) = pack8(x);
-      *(u32x4*)(dst + eb * 2) = pack8(x + 8);
+      if constexpr (OUT8) {
+        const float inv = kind == 0 ? a.q_inv_scale : a.k_inv_scale;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) x[i] *= inv;
+        *(u32x2*)(dst + ea) = pack8_e4m3(x);
+        *(u32x2*)(dst + eb) = pack8_e4m3(x + 8);
+      } else {
+        *(u32x4*)(dst + ea * 2) = pack8(x);
+        *(u32x4*)(dst + eb * 2) = pack8(x + 8);
+      }
     }
   }
 }
@@ -332,16 +361,24 @@ __global__ __launch_bounds__(THREADS) void rotary_kernel(const void* xin, const 
 hipError_t launch_prologue(const PrologueKernArgs& a_in, hipStream_t stream) {
   if (a_in.S <= 0) return hipSuccess;
   const PrologueKernArgs& a = a_in;
-  const int rows = a.Hq + 2 * a.Hkv;
+  const int rows = a.Hq + (a.out_fp8 ? 1 : 2) * a.Hkv;
   int tpb = 1;
   while (tpb < 8 && 2 * tpb * rows <= GROUPS) tpb *= 2;
   const dim3 grid((unsigned)((a.S + tpb - 1) / tpb)), block(THREADS);
+#define MAGI_PROLOGUE(TPB)                                                                  \
+  do {                                                                                      \
+    if (a.out_fp8)                                                                          \
+      hipLaunchKernelGGL((prologue_kernel<TPB, true>), grid, block, 0, stream, a);          \
+    else                                                                                    \
+      hipLaunchKernelGGL((prologue_kernel<TPB, false>), grid, block, 0, stream, a);         \
+  } while (0)
   switch (tpb) {
-    case 1: hipLaunchKernelGGL(prologue_kernel<1>, grid, block, 0, stream, a); break;
-    case 2: hipLaunchKernelGGL(prologue_kernel<2>, grid, block, 0, stream, a); break;
-    case 4: hipLaunchKernelGGL(prologue_kernel<4>, grid, block, 0, stream, a); break;
-    default: hipLaunchKernelGGL(prologue_kernel<8>, grid, block, 0, stream, a); break;
+    case 1: MAGI_PROLOGUE(1); break;
+    case 2: MAGI_PROLOGUE(2); break;
+    case 4: MAGI_PROLOGUE(4); break;
+    default: MAGI_PROLOGUE(8); break;
   }
+#undef MAGI_PROLOGUE
   return hipGetLastError();
 }
 

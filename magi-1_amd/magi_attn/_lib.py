@@ -47,6 +47,7 @@ class AttnArgs(C.Structure):
         ("out_group_heads", C.c_int32), ("o_stride_g", C.c_int64), ("score_bound", C.c_float),
         ("q_tile_rows", C.c_int32),
         ("q_norm_gamma", C.c_void_p), ("q_norm_beta", C.c_void_p), ("q_norm_eps", C.c_float), ("q_norm_kind", C.c_int32),
+        ("k2_scale", C.c_void_p), ("v2_scale", C.c_void_p),
     ]
 
 
@@ -60,11 +61,22 @@ class PrologueArgs(C.Structure):
         ("S", C.c_int32), ("n_cache_rows", C.c_int32),
         ("Hq", C.c_int32), ("Hkv", C.c_int32), ("D", C.c_int32), ("R2", C.c_int32),
         ("norm_kind", C.c_int32), ("eps", C.c_float), ("batch", C.c_int32), ("q_premul", C.c_float),
+        ("out_dtype", C.c_int32), ("q_quant_scale", C.c_float), ("k_quant_scale", C.c_float),
+    ]
+
+
+class QuantizeArgs(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p), ("x_stride_t", C.c_int64), ("x_stride_h", C.c_int64),
+        ("T", C.c_int32), ("H", C.c_int32), ("D", C.c_int32), ("chunk_tokens", C.c_int32),
+        ("premul", C.c_float), ("pow2_scales", C.c_int32),
+        ("y", C.c_void_p), ("scales", C.c_void_p), ("n_rows_first", C.c_int32),
+        ("y2", C.c_void_p), ("scales2", C.c_void_p),
     ]
 
 
 EXPORTS = ("magi_version", "magi_last_error", "magi_attn_fwd", "magi_qk_prologue", "magi_head_norm",
-           "magi_apply_rotary", "magi_quantize_fp8", "magi_layer_norm")
+           "magi_apply_rotary", "magi_quantize_fp8", "magi_quantize_fp8_split", "magi_layer_norm")
 
 _lib = None
 
@@ -96,6 +108,8 @@ def lib() -> C.CDLL:
         l.magi_quantize_fp8.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32,
                                         C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_int32, C.c_void_p]
         l.magi_quantize_fp8.restype = C.c_int
+        l.magi_quantize_fp8_split.argtypes = [C.POINTER(QuantizeArgs), C.c_void_p]
+        l.magi_quantize_fp8_split.restype = C.c_int
         _lib = l
     return _lib
 

@@ -80,6 +80,19 @@ class Fp8KVCache:
         self.v = torch.zeros_like(self.k)
         self.k_scale = torch.ones(n_chunks, num_query_groups, dtype=torch.float32, device=device)
         self.v_scale = torch.ones_like(self.k_scale)
+        self._k_const = None  # the value every row of k_scale holds, once a writer with constant K scales said so
+
+    def note_constant_k_scale(self, value: float, first_chunk: int, n_chunks: int) -> None:
+        """A writer whose K scale is one constant (the prologue with e4m3 outputs) is about to store chunks
+        [first_chunk, first_chunk + n_chunks).  While every writer uses the same constant the table is filled
+        once and never touched again; a different constant (the norm parameters changed while rows quantised
+        with the old one are still cached) only rewrites the rows of the chunks being stored."""
+        if self._k_const is None:
+            self.k_scale.fill_(value)
+            self._k_const = value
+        elif self._k_const != value:
+            self.k_scale[first_chunk:first_chunk + n_chunks].fill_(value)
+            self._k_const = float("nan")  # mixed from now on: every later store writes its rows
 
     @property
     def max_sequence_length(self) -> int:

@@ -15,6 +15,7 @@ used for device memory and the current stream only.
 from __future__ import annotations
 
 import ctypes as C
+import math
 from typing import Optional, Tuple
 
 import torch
@@ -64,6 +65,8 @@ def range_attention(
     q_scale: Optional[torch.Tensor] = None,
     k_scale: Optional[torch.Tensor] = None,
     v_scale: Optional[torch.Tensor] = None,
+    k2_scale: Optional[torch.Tensor] = None,
+    v2_scale: Optional[torch.Tensor] = None,
     scale_chunk_tokens: int = 0,
     fp8_pow2_prescaled: bool = False,
     q_prescaled: bool = False,
@@ -78,6 +81,9 @@ def range_attention(
 
     k and v may be strided views (e.g. the two halves of an interleaved KV cache); with
     k2 / v2 the key axis is the concatenation [k[:k_split] | k2] without copying.
+
+    k2_scale / v2_scale (fp8, with k2 / v2): the side segment's scale rows in tables of their own, row 0 = the chunk
+    that starts at k_split; without them k_scale / v_scale are indexed across k_split as one table.
 
     q_prescaled (bf16): q already carries softmax_scale * log2(e) (qk_prologue(..., q_premul=that)), so q . k is the
     exp2 exponent: the kernel skips its per-score multiply; softmax_scale is ignored.
@@ -124,6 +130,11 @@ def range_attention(
     a.out, a.lse = _ptr(out), _ptr(lse)
     a.q_ranges, a.k_ranges = _ptr(q_ranges), _ptr(k_ranges)
     a.q_scale, a.k_scale, a.v_scale = _ptr(q_scale), _ptr(k_scale), _ptr(v_scale)
+    for name, t in (("q_scale", q_scale), ("k_scale", k_scale), ("v_scale", v_scale), ("k2_scale", k2_scale),
+                    ("v2_scale", v2_scale)):
+        if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or t.device != q.device):
+            raise ValueError(f"{name} must be a contiguous fp32 tensor on q's device")
+    a.k2_scale, a.v2_scale = _ptr(k2_scale), _ptr(v2_scale)
     a.q_stride_t, a.q_stride_h = q.stride(0), q.stride(1)
     a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1)
     a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1)
@@ -270,6 +281,75 @@ def qk_prologue(q_raw, k_raw, v_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int,
     return q_out, kv_out, kv_tail
 
 
+def qk_prologue_fp8(q_raw, k_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int, q_scale: float, k_scale: float,
+                    eps: float = 1e-6, norm_kind: int = L.MAGI_NORM_LAYERNORM_1P, k_out: Optional[torch.Tensor] = None,
+                    n_cache_rows: Optional[int] = None, k_tail: Optional[torch.Tensor] = None,
+                    q_out: Optional[torch.Tensor] = None, batch: int = 1, q_premul: float = 1.0):
+    """qk_prologue with e4m3 outputs (magi_prologue_args.out_dtype): q [S, Hq, D] = sat_e4m3(q * q_premul / q_scale)
+    and K rows [*, Hkv, D] = sat_e4m3(k / k_scale) straight from the norm + rotary pass, with the two constant
+    scales of the call (powers of two; see pow2_scale_for).  k_out takes the first n_cache_rows tokens (a view of
+    an fp8 cache's K rows at the write position), k_tail the rest; with neither a fresh [S, Hkv, D] tensor.
+    V is not part of this pass (quantize_fp8_split takes it from the raw projection).
+    Returns (q8, k_out, k_tail)."""
+    S = q_raw.shape[0]
+    D = 128
+    dev = q_raw.device
+    f8 = torch.float8_e4m3fn
+    if q_out is None:
+        q_out = torch.empty((S, Hq, D), dtype=f8, device=dev)
+    if q_out.dtype != f8 or tuple(q_out.shape) != (S, Hq, D) or not q_out.is_contiguous():
+        raise ValueError("q_out must be a contiguous float8_e4m3fn [S, Hq, 128] tensor")
+    if k_out is None and k_tail is None:
+        k_out = torch.empty((S, Hkv, D), dtype=f8, device=dev)
+        n_cache_rows = S
+    if n_cache_rows is None:
+        n_cache_rows = S if k_tail is None else 0
+    for name, t in (("q_raw", q_raw), ("k_raw", k_raw)):
+        if t.dtype != torch.bfloat16 or t.stride(-1) != 1 or t.dim() != 2:
+            raise ValueError(f"{name} must be a 2-D bf16 tensor with contiguous rows")
+    for name, t in (("k_out", k_out), ("k_tail", k_tail)):
+        if t is not None and (t.dtype != f8 or t.dim() != 3 or t.shape[1:] != (Hkv, D) or t.stride(2) != 1
+                              or t.stride(1) != D):
+            raise ValueError(f"{name} must be float8_e4m3fn [rows, Hkv, D] with contiguous heads")
+    if k_out is not None and k_out.shape[0] < n_cache_rows:
+        raise ValueError("k_out is shorter than n_cache_rows")
+    if k_tail is not None and k_tail.shape[0] < S - n_cache_rows:
+        raise ValueError("k_tail is shorter than S - n_cache_rows")
+    f32 = lambda t: None if t is None else t.to(torch.float32).contiguous()
+    gq, bq, gk, bk = f32(gq), f32(bq), f32(gk), f32(bk)
+    a = L.PrologueArgs()
+    R2 = 0
+    if rope is not None:
+        if rope.dtype != torch.float32 or rope.dim() != 2 or rope.shape[0] * max(batch, 1) != S or not rope.is_contiguous():
+            raise ValueError("rope must be a contiguous fp32 [S / batch, 2*R2] tensor")
+        R2 = rope.shape[1] // 2
+    a.q_raw, a.k_raw, a.v_raw, a.rope = _ptr(q_raw), _ptr(k_raw), None, _ptr(rope)
+    a.gq, a.bq, a.gk, a.bk = _ptr(gq), _ptr(bq), _ptr(gk), _ptr(bk)
+    a.q_out, a.kv_out, a.kv_tail = _ptr(q_out), _ptr(k_out), _ptr(k_tail)
+    a.q_raw_stride_t, a.k_raw_stride_t = q_raw.stride(0), k_raw.stride(0)
+    a.kv_stride_t = 0 if k_out is None else k_out.stride(0)
+    a.kv_tail_stride_t = 0 if k_tail is None else k_tail.stride(0)
+    a.S, a.n_cache_rows = S, int(n_cache_rows)
+    a.Hq, a.Hkv, a.D, a.R2 = Hq, Hkv, D, R2
+    a.norm_kind, a.eps, a.batch = int(norm_kind), float(eps), int(batch)
+    a.q_premul = float(q_premul)
+    a.out_dtype = L.MAGI_DTYPE_FP8_E4M3
+    a.q_quant_scale, a.k_quant_scale = float(q_scale), float(k_scale)
+    with torch.cuda.device(dev):
+        L.check(L.lib().magi_qk_prologue(C.byref(a), _stream()))
+    return q_out, k_out, k_tail
+
+
+def pow2_scale_for(bound: float) -> float:
+    """Smallest power of two s with bound / s <= 448 (the largest e4m3 value): the scale to quantise values of
+    magnitude <= bound with.  e4m3 being a floating-point format, a bound that is a few times too large costs
+    no precision."""
+    if not (bound > 0.0) or bound == float("inf"):
+        raise ValueError("bound must be positive and finite")
+    m, e = math.frexp(bound / 448.0)  # bound / 448 = m * 2^e, 0.5 <= m < 1
+    return math.ldexp(1.0, e - 1 if m == 0.5 else e)
+
+
 def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[torch.Tensor], eps: float = 1e-5,
                out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """LayerNorm over the last axis of a bf16 tensor with fp32 statistics: the layer input norm of
@@ -346,3 +426,38 @@ def quantize_fp8(x: torch.Tensor, chunk_tokens: int, premul: float = 1.0, pow2_s
         L.check(L.lib().magi_quantize_fp8(x.data_ptr(), x.stride(0), x.stride(1), y.data_ptr(), scales.data_ptr(), T, H, D,
                                           int(chunk_tokens), float(premul), int(pow2_scales), _stream()))
     return y, scales
+
+
+def quantize_fp8_split(x: torch.Tensor, chunk_tokens: int, n_rows_first: int, out: Optional[torch.Tensor],
+                       scales_out: Optional[torch.Tensor], out2: Optional[torch.Tensor],
+                       scales2_out: Optional[torch.Tensor], premul: float = 1.0, pow2_scales: bool = False) -> None:
+    """quantize_fp8 in ONE launch with two destinations (magi_quantize_fp8_split): tokens below n_rows_first (a
+    multiple of chunk_tokens unless it is T) go to out / scales_out, e.g. the rows of an fp8 KV cache at the write
+    position and the matching rows of its scale table; the others to out2 / scales2_out, indexed from
+    n_rows_first.  Destinations are contiguous and at least as long as their share; a share of zero rows may
+    pass None."""
+    _check_thd(x, "x")
+    if x.dtype != torch.bfloat16:
+        raise TypeError("x must be bf16")
+    T, H, D = x.shape
+    n1 = int(n_rows_first)
+    if not (0 <= n1 <= T) or (n1 < T and n1 % chunk_tokens):
+        raise ValueError("n_rows_first must lie in [0, T] and, below T, be a multiple of chunk_tokens")
+    for name, y, sc, rows in (("out", out, scales_out, n1), ("out2", out2, scales2_out, T - n1)):
+        if rows == 0:
+            continue
+        chunks = (rows + chunk_tokens - 1) // chunk_tokens
+        if (y is None or y.dtype != torch.float8_e4m3fn or y.dim() != 3 or y.shape[0] < rows or tuple(y.shape[1:]) != (H, D)
+                or not y.is_contiguous() or y.device != x.device):
+            raise ValueError(f"{name} must be a contiguous float8_e4m3fn [>= {rows}, H, 128] tensor on x's device")
+        if (sc is None or sc.dtype != torch.float32 or sc.dim() != 2 or sc.shape[0] < chunks or sc.shape[1] != H
+                or not sc.is_contiguous() or sc.device != x.device):
+            raise ValueError(f"the scales of {name} must be a contiguous fp32 [>= {chunks}, H] tensor on x's device")
+    a = L.QuantizeArgs()
+    a.x, a.x_stride_t, a.x_stride_h = _ptr(x), x.stride(0), x.stride(1)
+    a.T, a.H, a.D, a.chunk_tokens = T, H, D, int(chunk_tokens)
+    a.premul, a.pow2_scales = float(premul), int(pow2_scales)
+    a.y, a.scales, a.n_rows_first = _ptr(out), _ptr(scales_out), n1
+    a.y2, a.scales2 = _ptr(out2), _ptr(scales2_out)
+    with torch.cuda.device(x.device):
+        L.check(L.lib().magi_quantize_fp8_split(C.byref(a), _stream()))

@@ -32,7 +32,8 @@ import math
 
 from . import _lib as L
 from .cache import Fp8KVCache
-from .functional import head_norm, layer_norm, qk_prologue, quantize_fp8, range_attention
+from .functional import (head_norm, layer_norm, pow2_scale_for, qk_prologue, qk_prologue_fp8, quantize_fp8_split,
+                         range_attention)
 from .params import InferenceParams, ModelMetaArgs, PackedCrossAttnParams
 
 
@@ -62,10 +63,20 @@ class FusedLayerNorm(torch.nn.Module):
 
     def gamma_beta_fp32(self) -> Tuple[torch.Tensor, torch.Tensor]:
         """(gamma - 1 form, beta) as the kernels take them.  weight + 1 is formed in the parameter
-        dtype first, as the reference does, so a bf16 parameter rounds the same way."""
-        w = self.weight.detach()
-        g = ((w + 1).float() - 1.0) if self.zero_centered_gamma else (w.float() - 1.0)
-        return g, self.bias.detach().float()
+        dtype first, as the reference does, so a bf16 parameter rounds the same way.  Converted once per set of
+        parameter values (no launches on later calls) and kept until a parameter is modified or replaced."""
+        # (a write through `.data` does not advance _version: callers that patch parameters that way call
+        # invalidate_cached_parameters())
+        key = tuple(x for t in (self.weight, self.bias) for x in (id(t), t._version, t.data_ptr(), t.dtype, t.device))
+        if self.__dict__.get("_gb_key") != key:
+            w = self.weight.detach()
+            g = ((w + 1).float() - 1.0) if self.zero_centered_gamma else (w.float() - 1.0)
+            self.__dict__["_gb"] = (g.contiguous(), self.bias.detach().float().contiguous())
+            self.__dict__["_gb_key"] = key
+        return self.__dict__["_gb"]
+
+    def invalidate_cached_parameters(self) -> None:
+        self.__dict__.pop("_gb_key", None)
 
     def output_norm_bound(self) -> float:
         """Upper bound of the Euclidean norm of any output row: the normalised row has norm <= sqrt(n) (exactly
@@ -233,24 +244,70 @@ class FullyParallelAttention(torch.nn.Module):
             raise ValueError("this layer's cache entry is not an Fp8KVCache with chunk_tokens == clip_token_nums")
         return cache
 
-    def _core_attention_fp8(self, q: torch.Tensor, kv_new: torch.Tensor, inference_params: Optional[InferenceParams],
+    def fp8_operand_scales(self) -> Tuple[float, float]:
+        """Constant power-of-two scales for the e4m3 forms of q (carrying softmax_scale * log2(e)) and k: no
+        element of a QK-normed row can exceed the row's length, which the norm parameters bound
+        (FusedLayerNorm.output_norm_bound) and the rotary embedding preserves, so these scales never saturate and
+        the prologue can quantise without an absmax pass.  Cached like score_bounds()."""
+        lns = (self.q_layernorm, self.k_layernorm)
+        key = tuple((id(t), t._version) for ln in lns for t in (ln.weight, ln.bias))
+        if getattr(self, "_fp8_scales_key", None) != key:
+            nq, nk = (ln.output_norm_bound() for ln in lns)
+            self._fp8_scales = (pow2_scale_for(self._q_premul * nq), pow2_scale_for(nk))
+            self._fp8_scales_key = key
+        return self._fp8_scales
+
+    def _const_scale_table(self, value: float, rows: int, heads: int, device) -> torch.Tensor:
+        """[rows, heads] fp32 filled with `value`, kept between calls (a launch only when it has to grow)."""
+        tabs = self.__dict__.setdefault("_const_tabs", {})
+        key = (value, heads, str(device))
+        t = tabs.get(key)
+        if t is None or t.shape[0] < rows:
+            if len(tabs) > 8:
+                tabs.clear()
+            t = torch.full((max(rows, 16), heads), value, dtype=torch.float32, device=device)
+            tabs[key] = t
+        return t[:rows]
+
+    def _side_buffer(self, name: str, shape, dtype, device) -> torch.Tensor:
+        """A per-layer buffer for rows that must not be persisted, kept between calls."""
+        t = getattr(self, name, None)
+        if t is None or t.shape[0] < shape[0] or t.shape[1:] != tuple(shape[1:]) or t.dtype != dtype or t.device != device:
+            t = torch.empty(shape, dtype=dtype, device=device)
+            setattr(self, name, t)
+        return t[:shape[0]]
+
+    def _core_attention_fp8(self, raw, rope: torch.Tensor, inference_params: Optional[InferenceParams],
                             meta_args: ModelMetaArgs, use_cache: bool, out: Optional[torch.Tensor]) -> torch.Tensor:
-        """Self-attention on e4m3 operands: q [S, Hq, D] and kv_new [S, Hkv, 2D] are the prologue's bf16 results.
+        """Self-attention on e4m3 operands, three launches from the raw projections (q_raw, k_raw, v_raw) on: the
+        prologue writes q and k as e4m3 with the constant scales of fp8_operand_scales(), k straight into the
+        cache rows; one quantiser launch takes v's per-(chunk, head) absmax scales and writes v; the attention.
         Scale chunks are video chunks (clip_token_nums tokens), so the cache rules of the bf16 path
         (dit_module.py:905-931: append at slice_point, keep nothing when update_kv_cache is False, keep all but
         the last chunk under distill_nearly_clean_chunk) carry over chunk by chunk."""
         D = self.hidden_size_per_attention_head
+        Hq, Hkv = self.num_attention_heads, self.num_query_groups_per_partition
         Lc = meta_args.clip_token_nums
         p = meta_args.core_attn_params
-        S = q.shape[0]
-        q8, qs = quantize_fp8(q, Lc, premul=D ** -0.5 * math.log2(math.e), pow2_scales=True)
-        k_new, v_new = kv_new[..., :D], kv_new[..., D:]
-        kw = dict(q_scale=qs, scale_chunk_tokens=Lc, fp8_pow2_prescaled=True, out=out, return_lse=False)
+        q_raw, k_raw, v_raw = (t.reshape(t.shape[0] * t.shape[1], -1) for t in raw)
+        S = q_raw.shape[0]
+        dev = q_raw.device
+        n_chunks = (S + Lc - 1) // Lc
+        v3 = v_raw.view(S, Hkv, D)
+        qs_c, ks_c = self.fp8_operand_scales()
+        gq, bq = self.q_layernorm.gamma_beta_fp32()
+        gk, bk = self.k_layernorm.gamma_beta_fp32()
+        pro = dict(Hq=Hq, Hkv=Hkv, q_scale=qs_c, k_scale=ks_c, eps=self.eps, q_premul=self._q_premul)
+        kw = dict(q_scale=self._const_scale_table(qs_c, n_chunks, Hq, dev), scale_chunk_tokens=Lc,
+                  fp8_pow2_prescaled=True, out=out, return_lse=False)
+        f8 = torch.float8_e4m3fn
         if not use_cache:
-            k8, ks = quantize_fp8(k_new, Lc, pow2_scales=True)
-            v8, vs = quantize_fp8(v_new, Lc, pow2_scales=True)
-            o, _ = range_attention(q8, k8, v8, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k, k_scale=ks, v_scale=vs,
-                                   **kw)
+            q8, k8, _ = qk_prologue_fp8(q_raw, k_raw, rope, gq, bq, gk, bk, **pro)
+            v8 = torch.empty((S, Hkv, D), dtype=f8, device=dev)
+            vs = torch.empty((n_chunks, Hkv), dtype=torch.float32, device=dev)
+            quantize_fp8_split(v3, Lc, S, v8, vs, None, None, pow2_scales=True)
+            o, _ = range_attention(q8, k8, v8, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
+                                   k_scale=self._const_scale_table(ks_c, n_chunks, Hkv, dev), v_scale=vs, **kw)
             return o
         cache = self._cache_fp8(inference_params, Lc)
         start = meta_args.slice_point * Lc
@@ -263,22 +320,26 @@ class FullyParallelAttention(torch.nn.Module):
         if start + n_keep > cache.max_sequence_length:
             raise ValueError("KV cache overflow")
         c0 = start // Lc
+        n_side = S - n_keep
+        k_side = v_side = vs_side = None
+        if n_side:
+            k_side = self._side_buffer("_k8_side", (n_side, Hkv, D), f8, dev)
+            v_side = self._side_buffer("_v8_side", (n_side, Hkv, D), f8, dev)
+            vs_side = self._side_buffer("_v8_side_scale", (n_side // Lc, Hkv), torch.float32, dev)
         if n_keep:
-            rows, chunks = slice(start, start + n_keep), slice(c0, c0 + n_keep // Lc)
-            quantize_fp8(k_new[:n_keep], Lc, pow2_scales=True, out=cache.k[rows], scales_out=cache.k_scale[chunks])
-            quantize_fp8(v_new[:n_keep], Lc, pow2_scales=True, out=cache.v[rows], scales_out=cache.v_scale[chunks])
+            cache.note_constant_k_scale(ks_c, c0, n_keep // Lc)
+        q8, _, _ = qk_prologue_fp8(q_raw, k_raw, rope, gq, bq, gk, bk, k_out=cache.k[start:], n_cache_rows=n_keep,
+                                   k_tail=k_side, **pro)
+        quantize_fp8_split(v3, Lc, n_keep, cache.v[start:], cache.v_scale[c0:], v_side, vs_side, pow2_scales=True)
         split = start + n_keep
-        if n_keep == S:
+        if not n_side:
             o, _ = range_attention(q8, cache.k[:split], cache.v[:split], p.q_range, p.k_range, p.max_seqlen_q,
                                    p.max_seqlen_k, k_scale=cache.k_scale, v_scale=cache.v_scale, **kw)
             return o
-        # rows that must not be persisted: a side buffer behind the cached prefix, its scales behind the prefix's
-        k2, k2s = quantize_fp8(k_new[n_keep:], Lc, pow2_scales=True)
-        v2, v2s = quantize_fp8(v_new[n_keep:], Lc, pow2_scales=True)
-        ks = torch.cat([cache.k_scale[:split // Lc], k2s])
-        vs = torch.cat([cache.v_scale[:split // Lc], v2s])
+        # rows that must not be persisted: side buffers behind the cached prefix, with scale tables of their own
         o, _ = range_attention(q8, cache.k[:split], cache.v[:split], p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                               k2=k2, v2=v2, k_split=split, k_scale=ks, v_scale=vs, **kw)
+                               k2=k_side, v2=v_side, k_split=split, k_scale=cache.k_scale, v_scale=cache.v_scale,
+                               k2_scale=self._const_scale_table(ks_c, n_side // Lc, Hkv, dev), v2_scale=vs_side, **kw)
         return o
 
     # --------------------------------------------------- reference-shaped pieces
@@ -503,8 +564,8 @@ class FullyParallelAttention(torch.nn.Module):
         if self.attention_dtype == "fp8":
             if bs != 1 or (use_cache and inference_params.max_batch_size != 1):
                 raise ValueError("the fp8 self-attention runs at batch 1")
-            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw, rope=rope)
-            core = self._core_attention_fp8(q, kv, inference_params, meta_args, use_cache, core_dst)
+            rope8 = rope if rope is not None else torch.cat([sin_emb, cos_emb], dim=-1).float().contiguous()
+            core = self._core_attention_fp8(raw, rope8, inference_params, meta_args, use_cache, core_dst)
         elif not use_cache:
             q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw, q_premul=self._q_premul, rope=rope)
             core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst, q_prescaled=True,

@@ -155,7 +155,8 @@ def apply_rope_neox_partial(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tenso
 # --------------------------------------------------------------------------------------
 def prologue(q_raw: torch.Tensor, k_raw: torch.Tensor, v_raw: torch.Tensor, rope: torch.Tensor,
              gq: torch.Tensor, bq: torch.Tensor, gk: torch.Tensor, bk: torch.Tensor,
-             eps: float = 1e-6, norm: str = "layernorm_1p", q_premul: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+             eps: float = 1e-6, norm: str = "layernorm_1p", q_premul: float = 1.0,
+             downcast: bool = True) -> Tuple[torch.Tensor, torch.Tensor]:
     """q_raw [S, Hq, D], k_raw / v_raw [S, Hkv, D] in bf16 (the projections' outputs, batch 1).
 
     q_premul (no counterpart in the reference; 1.0 reproduces it): factor applied to q in fp32 ahead of the
@@ -164,6 +165,9 @@ def prologue(q_raw: torch.Tensor, k_raw: torch.Tensor, v_raw: torch.Tensor, rope
     Returns (q [S, Hq, D] bf16, kv [S, Hkv, 2D] bf16) as get_q (:953-963) and get_kv (:991-996)
     do: upcast to fp32, norm, rotary in fp32, downcast to the input dtype; V is only
     re-laid-out; kv = cat([k, v], -1).  sin is the first half of the table (:1147).
+
+    downcast=False (no counterpart in the reference) stops ahead of the downcast and returns (q, k) in fp32: what
+    a quantiser that reads the norm + rotary result without a bf16 intermediate sees.
     """
     sin, cos = rope.tensor_split(2, -1)
 
@@ -178,10 +182,12 @@ def prologue(q_raw: torch.Tensor, k_raw: torch.Tensor, v_raw: torch.Tensor, rope
         xf = apply_rope_neox_partial(xf, cos.float(), sin.float())
         if premul != 1.0:
             xf = xf * premul
-        return xf.to(x.dtype)
+        return xf.to(x.dtype) if downcast else xf
 
     q = one(q_raw, gq, bq, q_premul)
     k = one(k_raw, gk, bk)
+    if not downcast:
+        return q, k
     return q, torch.cat([k, v_raw], dim=-1)
 
 

@@ -12,6 +12,7 @@ normalised Q / K): cosine >= 0.998 and max-abs <= 2^-5 * max|V| (an output row i
 of V rows, e4m3 rounds a value v to within 2^-4 |v|; half of that bound, which also has to absorb the
 score errors, holds on every seeded case here; at benchmark sizes the averaging over ~10^5 keys brings
 max-abs below 1e-2).  Against the dequantised-input oracle: max-abs <= 4e-2 and cosine >= 0.9995."""
+import math
 import os
 
 import numpy as np
@@ -48,6 +49,76 @@ def test_quantiser_bit_exact_with_oracle(dev):
     assert torch.equal(y2.cpu().view(torch.uint8), y2r.view(torch.uint8)) and torch.equal(s2.cpu(), s2r)
     z, sz = M.quantize_fp8(torch.zeros(10, 1, 128, dtype=torch.bfloat16, device=dev), 10)
     assert torch.all(z.float() == 0) and torch.all(sz > 0)
+
+
+def test_one_launch_quantiser_with_two_destinations(dev):
+    """magi_quantize_fp8_split: bytes and scales equal to the oracle's quantiser on each share (so also to the
+    multi-launch form), written at the right rows of two destinations and nowhere else; strided input; a group
+    size above the one-launch limit of magi_quantize_fp8 gives the same bytes through either entry point."""
+    g = torch.Generator().manual_seed(3)
+    C, H, D = 48, 3, 128
+    for n_chunks, keep in ((5, 3), (4, 4), (3, 0), (1, 1)):
+        T = n_chunks * C
+        big = (torch.randn(T, 2 * H * D, generator=g) * 3).bfloat16()
+        x = big.view(T, H, 2 * D)[..., D:]  # the V half of an interleaved projection
+        n1 = keep * C
+        y1 = torch.zeros(n1 + 7, H, D, device=dev).to(torch.float8_e4m3fn)
+        s1 = torch.full((keep + 2, H), -1.0, device=dev)
+        y2 = torch.zeros(T - n1 + 3, H, D, device=dev).to(torch.float8_e4m3fn)
+        s2 = torch.full((n_chunks - keep + 1, H), -1.0, device=dev)
+        M.quantize_fp8_split(x.to(dev), C, n1, y1, s1, y2, s2, pow2_scales=True)
+        y_ref, s_ref = O.quantize_per_head_chunk(x, C, pow2=True)
+        u8 = lambda t: t.cpu().view(torch.uint8)
+        assert torch.equal(u8(y1[:n1]), u8(y_ref[:n1])) and torch.equal(u8(y2[:T - n1]), u8(y_ref[n1:]))
+        assert torch.equal(s1[:keep].cpu(), s_ref[:keep]) and torch.equal(s2[:n_chunks - keep].cpu(), s_ref[keep:])
+        assert torch.all(y1[n1:].float() == 0) and torch.all(y2[T - n1:].float() == 0)
+        assert torch.all(s1[keep:] == -1) and torch.all(s2[n_chunks - keep:] == -1)
+    # ragged last chunk, non-power-of-two scales, premul
+    x = torch.randn(100, 2, D, generator=g).bfloat16()
+    y = torch.empty(100, 2, D, device=dev).to(torch.float8_e4m3fn)
+    sc = torch.empty(3, 2, device=dev)
+    M.quantize_fp8_split(x.to(dev), 40, 100, y, sc, None, None, premul=0.3)
+    y_ref, s_ref = O.quantize_per_head_chunk(x, 40, premul=0.3)
+    assert torch.equal(y.cpu().view(torch.uint8), y_ref.view(torch.uint8)) and torch.equal(sc.cpu(), s_ref)
+    # one group of 9000 tokens: magi_quantize_fp8 takes its multi-launch form, the split entry point one launch
+    x = torch.randn(9000, 1, D, generator=g).bfloat16().to(dev)
+    ya, sa = M.quantize_fp8(x, 9000, pow2_scales=True)
+    yb = torch.empty_like(ya)
+    sb = torch.empty_like(sa)
+    M.quantize_fp8_split(x, 9000, 9000, yb, sb, None, None, pow2_scales=True)
+    assert torch.equal(ya.view(torch.uint8), yb.view(torch.uint8)) and torch.equal(sa, sb)
+    with pytest.raises(ValueError):
+        M.quantize_fp8_split(x, 4000, 100, ya, sa, yb, sb)  # split inside a chunk
+
+
+def test_fp8_side_segment_with_scale_tables_of_its_own(dev):
+    """k2_scale / v2_scale: the side segment's scales in separate tables give the bytes of the call that indexes
+    one concatenated table, in both scale modes; the cache's own table rows behind k_split (here poisoned) are
+    not read."""
+    L, dn, sp, Hq, Hkv, D = 96, 3, 2, 4, 2, 128
+    Tq, Tk = dn * L, (sp + dn) * L
+    q, k, v = O.synthetic_qkv(Tq, Tk, Hq, Hkv, D, seed=21)
+    qr = torch.tensor(O.q_ranges_for(dn, L), dtype=torch.int32, device=dev)
+    kr = torch.tensor(O.default_kvrange(sp, dn, L), dtype=torch.int32, device=dev)
+    cs = D ** -0.5 * math.log2(math.e)
+    for pow2 in (False, True):
+        q8, qs = M.quantize_fp8(q.to(dev), L, premul=cs if pow2 else 1.0, pow2_scales=pow2)
+        k8, ks = M.quantize_fp8(k.to(dev), L, pow2_scales=pow2)
+        v8, vs = M.quantize_fp8(v.to(dev), L, pow2_scales=pow2)
+        kw = dict(q_scale=qs, scale_chunk_tokens=L, fp8_pow2_prescaled=pow2, return_lse=True)
+        want, lse_want = M.range_attention(q8, k8, v8, qr, kr, L, Tk, k_scale=ks, v_scale=vs, **kw)
+        for split_chunk in (0, 1, 3, 4):
+            split = split_chunk * L
+            ks_main, vs_main = ks.clone(), vs.clone()
+            ks_main[split_chunk:] = float("nan")
+            vs_main[split_chunk:] = float("nan")
+            got, lse = M.range_attention(q8, k8[:split], v8[:split], qr, kr, L, Tk, k2=k8[split:].clone(),
+                                         v2=v8[split:].clone(), k_split=split, k_scale=ks_main, v_scale=vs_main,
+                                         k2_scale=ks[split_chunk:].clone(), v2_scale=vs[split_chunk:].clone(), **kw)
+            assert torch.equal(got, want) and torch.equal(lse, lse_want), (pow2, split_chunk)
+    with pytest.raises(M.MagiError):  # a split inside a scale chunk cannot carry tables of its own
+        M.range_attention(q8, k8[:50], v8[:50], qr, kr, L, Tk, k2=k8[50:].clone(), v2=v8[50:].clone(), k_split=50,
+                          k_scale=ks, v_scale=vs, k2_scale=ks, v2_scale=vs, **kw)
 
 
 @pytest.mark.parametrize("L,dn,sp,Hq,Hkv,C", [(128, 1, 0, 1, 1, 128), (64, 2, 0, 2, 1, 64), (200, 3, 1, 6, 2, 200),

@@ -19,6 +19,8 @@ pytestmark = pytest.mark.gpu
 
 def _cosine(a, b):
     x, y = a.detach().double().cpu().flatten(), b.detach().double().cpu().flatten()
+    if x.norm() == 0 and y.norm() == 0:  # e.g. the cross attention of a batch row without text
+        return 1.0
     return (torch.dot(x, y) / (x.norm() * y.norm()).clamp_min(1e-30)).item()
 
 
@@ -57,6 +59,74 @@ def test_prologue_parity(dev, T, H, W, sp, dn, Hq, Hkv):
     _ulp_check(q, q_ref, "q")
     _ulp_check(kv[..., :D], kv_ref[..., :D], "k")
     assert torch.equal(kv[..., D:].cpu(), kv_ref[..., D:])  # V is a copy: bit exact
+
+
+def _e4m3_check(got, ref, what=""):
+    """got / ref float8_e4m3fn: equal but for values on a rounding boundary, which the different summation order of
+    the fp32 norm may push to the neighbouring code (bar: the neighbour at most, fewer than 2 in 1000 elements)."""
+    gb, rb = got.cpu().view(torch.uint8).int(), ref.cpu().view(torch.uint8).int()
+    assert gb.shape == rb.shape
+    if gb.numel() == 0:
+        return
+    diff = gb != rb
+    assert diff.float().mean().item() < 2e-3, f"{what}: {diff.float().mean().item():.2e} of the elements differ"
+    # neighbouring codes: same sign and magnitude codes one apart, or +-0 against the smallest subnormal
+    mag_g, mag_r = gb & 0x7f, rb & 0x7f
+    near = ((gb & 0x80) == (rb & 0x80)) & ((mag_g - mag_r).abs() <= 1) | ((mag_g + mag_r) <= 1)
+    assert torch.all(near | ~diff), f"{what}: more than one e4m3 code off"
+
+
+@pytest.mark.parametrize("T,H,W,sp,dn,Hq,Hkv,keep", [(2, 4, 6, 0, 2, 6, 2, 1), (6, 5, 7, 2, 3, 24, 8, 3), (4, 3, 3, 1, 2, 48, 8, 0),
+                                                     (1, 3, 3, 0, 1, 2, 1, 1), (3, 5, 3, 1, 3, 6, 1, 2)])
+def test_prologue_e4m3_outputs(dev, T, H, W, sp, dn, Hq, Hkv, keep):
+    """out_dtype e4m3: q and k leave the norm + rotary pass quantised with constant power-of-two scales, K straight
+    into the rows of an fp8 cache (first `keep` chunks) and a side buffer (the rest).  Expected values: the
+    oracle's prologue stopped ahead of its downcast, through the oracle's saturating e4m3 quantiser.  The scales
+    come from the norm-parameter bound (nothing saturates); a second run with a scale 64 times too small checks
+    the saturation to +-448."""
+    import math
+
+    S, D = T * H * W, 128
+    L = S // dn
+    cs = D ** -0.5 * math.log2(math.e)
+    qr, kr, vr, (gq, bq, gk, bk) = _inputs(S, Hq, Hkv, seed=S + Hq + 1)
+    rope = O.rope_for_forward(T, H, W, sp, dn)
+    q_f, k_f = O.prologue(qr.view(S, Hq, D), kr.view(S, Hkv, D), vr.view(S, Hkv, D), rope, gq, bq, gk, bk, q_premul=cs,
+                          downcast=False)
+    bound = lambda g, b: math.sqrt(D) * (g + 1).abs().max().item() + b.norm().item()
+    to = lambda t: t.to(dev)
+    for shrink in (1.0, 64.0):
+        qs = M.pow2_scale_for(cs * bound(gq, bq)) / shrink
+        ks = M.pow2_scale_for(bound(gk, bk)) / shrink
+        if shrink == 1.0:
+            assert (q_f.abs().max() / qs <= 448) and (k_f.abs().max() / ks <= 448)
+        cache_k = torch.zeros(S + 5, Hkv, D, device=dev).to(torch.float8_e4m3fn)
+        side = torch.zeros(S, Hkv, D, device=dev).to(torch.float8_e4m3fn)
+        n_keep = keep * L
+        q8, k_out, k_tail = M.qk_prologue_fp8(to(qr), to(kr), to(rope), to(gq), to(bq), to(gk), to(bk), Hq=Hq, Hkv=Hkv,
+                                              q_scale=qs, k_scale=ks, q_premul=cs, k_out=cache_k[5:], n_cache_rows=n_keep,
+                                              k_tail=side)
+        q_ref = O.quantize_e4m3(q_f, torch.tensor(qs))
+        k_ref = O.quantize_e4m3(k_f, torch.tensor(ks))
+        _e4m3_check(q8, q_ref, "q")
+        _e4m3_check(cache_k[5:5 + n_keep], k_ref[:n_keep], "k (cache rows)")
+        _e4m3_check(side[:S - n_keep], k_ref[n_keep:], "k (side rows)")
+        assert torch.all(cache_k[:5].float() == 0) and torch.all(cache_k[5 + n_keep:].float() == 0)
+        assert torch.all(side[S - n_keep:].float() == 0)
+        assert not torch.isnan(q8.float()).any() and not torch.isnan(cache_k.float()).any()
+        if shrink > 1.0:
+            assert q8.float().abs().max() == 448
+    # fresh outputs, strided raw rows (views of one projection result), no rotary, RMS norm
+    big = torch.randn(S, (Hq + 2 * Hkv) * D + 64, generator=torch.Generator().manual_seed(5)).bfloat16().to(dev)
+    qv, kv_ = big[:, :Hq * D], big[:, Hq * D:(Hq + Hkv) * D]
+    q8, k8, _ = M.qk_prologue_fp8(qv, kv_, None, to(gq), None, to(gk), None, Hq=Hq, Hkv=Hkv, q_scale=2.0 ** -4,
+                                  k_scale=2.0 ** -5, norm_kind=M.MAGI_NORM_RMSNORM_1P)
+    qn = O.rmsnorm(qv.cpu().view(S, Hq, D).float(), gq + 1)
+    kn = O.rmsnorm(kv_.cpu().view(S, Hkv, D).float(), gk + 1)
+    _e4m3_check(q8, O.quantize_e4m3(qn, torch.tensor(2.0 ** -4)), "q rms")
+    _e4m3_check(k8, O.quantize_e4m3(kn, torch.tensor(2.0 ** -5)), "k rms")
+    with pytest.raises(M.MagiError):
+        M.qk_prologue_fp8(qv, kv_, None, to(gq), None, to(gk), None, Hq=Hq, Hkv=Hkv, q_scale=0.0, k_scale=1.0)
 
 
 def test_prologue_folds_a_factor_into_q_ahead_of_the_rounding(dev):
@@ -429,6 +499,58 @@ def test_layer_with_fp8_self_attention_and_fp8_cache(dev):
             for got, ref_half in ((cache.k[rows].float() * sc(cache.k_scale), want[..., :D]),
                                   (cache.v[rows].float() * sc(cache.v_scale), want[..., D:])):
                 assert ((got - ref_half).abs() <= ref_half.abs() * 2 ** -4 + 2 ** -9 * ref_half.abs().max()).all()
+
+
+def test_fp8_layer_prepares_its_operands_in_two_launches(dev):
+    """Between the projection GEMM and the fp8 attention kernel the layer issues exactly two kernels: the prologue
+    with e4m3 outputs (q, and k into the cache rows) and the one-launch V quantiser; no absmax / conversion
+    passes and no torch elementwise kernels.  Read from a kernel trace of one steady-state forward (skipped when
+    the profiler records no device activity)."""
+    from torch.profiler import ProfilerActivity, profile
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+
+    hidden, Hq, Hkv, D = 256, 8, 2, 128
+    fr, H, W = 2, 3, 4
+    L = fr * H * W
+    torch.manual_seed(11)
+    layer = MOD.FullyParallelAttention(hidden, Hq, Hkv, layer_number=0, device=dev, attention_dtype="fp8")
+    rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
+    ip = P.InferenceParams(1, 6 * L)
+    g = torch.Generator().manual_seed(12)
+
+    def step(sp, dn, update, distill):
+        S = dn * L
+        hs = torch.randn(S, 1, hidden, generator=g).bfloat16().to(dev)
+        mask = torch.ones(dn, 1, 1, 8)
+        y = (torch.randn(dn * 8, hidden, generator=g) * 0.5).bfloat16().to(dev)
+        meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=sp, denoising_range_num=dn,
+                               range_num=sp + dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=True,
+                               distill_nearly_clean_chunk=distill, clip_token_nums=L, enable_cuda_graph=False,
+                               core_attn_params=P.build_core_attn_params(
+                                   R.q_ranges_from_chunks(dn, L).to(dev), R.generate_default_kvrange(sp, dn, L).to(dev), L),
+                               cross_attn_params=P.build_cross_attn_params(mask.to(dev), L, 8))
+        rope = rope_mod.get_embed_for_forward(dn * fr, H, W, sp, dn)
+        ip.update_kv_cache = update
+        with torch.no_grad():
+            return layer(hs, y, ip, rope, meta, proj_layout=True)
+
+    step(0, 2, True, False)  # warm-up: caches the fp32 norm parameters, the constant scale tables, the side buffers
+    step(0, 3, True, True)
+    torch.cuda.synchronize()
+    for args in ((1, 3, True, True), (2, 3, True, False)):  # with and without rows that are not persisted
+        with profile(activities=[ProfilerActivity.CUDA]) as prof:
+            step(*args)
+            torch.cuda.synchronize()
+        evs = sorted((e for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA and "Memcpy" not in e.name
+                      and "Memset" not in e.name), key=lambda e: e.time_range.start)
+        names = [e.name for e in evs]
+        if not names:
+            pytest.skip("the profiler recorded no device activity")
+        attn = [i for i, n in enumerate(names) if "attn_fwd_fp8_kernel" in n]
+        assert len(attn) == 1, names
+        gemm = max(i for i, n in enumerate(names[:attn[0]]) if n.startswith("Cijk_"))
+        between = names[gemm + 1:attn[0]]
+        assert len(between) == 2 and "prologue_kernel" in between[0] and "quantize_groups_kernel" in between[1], between
 
 
 # ----------------------------------------------------------------------------- layer input norm

@@ -502,7 +502,7 @@ def test_layer_with_fp8_self_attention_and_fp8_cache(dev):
 
 
 def test_fp8_layer_prepares_its_operands_in_two_launches(dev):
-    """Between the projection GEMM and the fp8 attention kernel the layer issues exactly two kernels: the prologue
+    """Between the GEMM of the projections and the fp8 attention kernel the layer issues exactly two kernels: the prologue
     with e4m3 outputs (q, and k into the cache rows) and the one-launch V quantiser; no absmax / conversion
     passes and no torch elementwise kernels.  Read from a kernel trace of one steady-state forward (skipped when
     the profiler records no device activity)."""
@@ -548,9 +548,10 @@ def test_fp8_layer_prepares_its_operands_in_two_launches(dev):
             pytest.skip("the profiler recorded no device activity")
         attn = [i for i, n in enumerate(names) if "attn_fwd_fp8_kernel" in n]
         assert len(attn) == 1, names
-        gemm = max(i for i, n in enumerate(names[:attn[0]]) if n.startswith("Cijk_"))
-        between = names[gemm + 1:attn[0]]
-        assert len(between) == 2 and "prologue_kernel" in between[0] and "quantize_groups_kernel" in between[1], between
+        ln = max(i for i, n in enumerate(names[:attn[0]]) if "layer_norm_kernel" in n)
+        between = names[ln + 1:attn[0]]  # the one GEMM of the four projections, then the two launches
+        assert len(between) == 3 and "magi::" not in between[0], between
+        assert "prologue_kernel" in between[1] and "quantize_groups_kernel" in between[2], between
 
 
 # ----------------------------------------------------------------------------- layer input norm

@@ -340,7 +340,7 @@ int magi_apply_rotary(const void* x, const float* cos, const float* sin, void* y
   return MAGI_OK;
 }
 
-int magi_quantize_fp8_split(const magi_quantize_args* p, void* stream) {
+static int quantize_impl(const magi_quantize_args* p, void* stream, bool always_one_launch) {
   if (!p) return fail(MAGI_EINVAL, "magi_quantize_fp8: args is NULL");
   if (p->D != 128) return fail(MAGI_ENOSYS, "magi_quantize_fp8: head_dim %d not implemented (128 only)", p->D);
   if (p->T < 0 || p->H < 0 || p->chunk_tokens <= 0) return fail(MAGI_EINVAL, "magi_quantize_fp8: bad size");
@@ -361,10 +361,12 @@ int magi_quantize_fp8_split(const magi_quantize_args* p, void* stream) {
   hipError_t e = magi::launch_quantize_fp8(static_cast<const char*>(p->x), p->x_stride_t * 2, p->x_stride_h * 2,
                                            static_cast<char*>(p->y), p->scales, p->T, p->H, p->chunk_tokens, p->premul,
                                            p->pow2_scales, p->n_rows_first, static_cast<char*>(p->y2), p->scales2,
-                                           static_cast<hipStream_t>(stream));
+                                           always_one_launch, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_quantize_fp8 launch");
   return MAGI_OK;
 }
+
+int magi_quantize_fp8_split(const magi_quantize_args* p, void* stream) { return quantize_impl(p, stream, true); }
 
 int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, void* y, float* scales, int32_t T,
                       int32_t H, int32_t D, int32_t chunk_tokens, float premul, int32_t pow2_scales, void* stream) {
@@ -382,7 +384,7 @@ int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, voi
   q.y = y;
   q.scales = scales;
   q.n_rows_first = T;
-  return magi_quantize_fp8_split(&q, stream);
+  return quantize_impl(&q, stream, false);
 }
 
 }  // extern "C"

@@ -558,11 +558,15 @@ __global__ __launch_bounds__(QT) void quantize_kernel(const char* x, long xs_t, 
   *(u32x2*)(y + row * 128 + part * 8) = quantize8(v, premul, sc);
 }
 
-// The whole job in one launch, for groups small enough that one workgroup can walk them twice (a video chunk of
-// one head is 0.4 MB at the 720p shape and stays in L2 between the passes): workgroup (h, c) takes the absmax of
-// its (chunk, head) group, reduces it through LDS, writes the scale, and quantises the group with it.  No memory
-// beyond the inputs and outputs.  Groups that start at or after token n_first go to the second destination.
+// The whole job in one launch with no memory beyond the inputs and outputs: a workgroup takes the absmax of its
+// (chunk, head) group (a video chunk of one head is 5.5 MB at the 720p shape), reduces it through LDS, and
+// quantises with the resulting scale.  To fill the chip when there are few groups, gridDim.z workgroups share a
+// group: each of them takes the absmax of the WHOLE group (a maximum does not depend on the order, so all arrive
+// at the same scale; the repeated reads are served by the caches, HBM sees the group once) and quantises its own
+// slice of the rows; slice 0 writes the scale.  Groups that start at or after token n_first go to the second
+// destination.
 constexpr int QT1 = 1024;
+constexpr int QROWS = QT1 / 16;  // rows per pass of a workgroup
 __global__ __launch_bounds__(QT1) void quantize_groups_kernel(const char* x, long xs_t, long xs_h, char* y, float* scales,
                                                               int T, int H, int chunk_tokens, float premul, int pow2,
                                                               int n_first, char* y2, float* scales2) {
@@ -572,14 +576,23 @@ __global__ __launch_bounds__(QT1) void quantize_groups_kernel(const char* x, lon
   const int lane16 = threadIdx.x & 15, sub = threadIdx.x >> 4;
   const char* const xcol = x + (long)h * xs_h + lane16 * 16;
   unsigned m = 0u;
-  for (int t = t_begin + sub; t < t_end; t += QT1 / 16) {
-    const u32x4 v = *(const u32x4*)(xcol + (long)t * xs_t);
+  auto fold = [&](const u32x4 v) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       m = max(m, (v[j] << 16) & 0x7fffffffu);
       m = max(m, v[j] & 0x7fff0000u);
     }
+  };
+  constexpr int UN = 8;  // loads in flight per lane
+  int t = t_begin + sub;
+  for (; t + (UN - 1) * QROWS < t_end; t += UN * QROWS) {
+    u32x4 v[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) v[u] = *(const u32x4*)(xcol + (long)(t + u * QROWS) * xs_t);
+#pragma unroll
+    for (int u = 0; u < UN; ++u) fold(v[u]);
   }
+  for (; t < t_end; t += QROWS) fold(*(const u32x4*)(xcol + (long)t * xs_t));
 #pragma unroll
   for (int o = 32; o >= 1; o >>= 1) m = max(m, (unsigned)__shfl_xor((int)m, o));
   if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = m;
@@ -589,12 +602,21 @@ __global__ __launch_bounds__(QT1) void quantize_groups_kernel(const char* x, lon
   const float sc = scale_of_absmax(__builtin_bit_cast(float, m), premul, pow2);
   const bool second = t_begin >= n_first;
   const int t_off = second ? n_first : 0;
-  if (threadIdx.x == 0) (second ? scales2 : scales)[(long)(c - t_off / chunk_tokens) * H + h] = sc;
-  char* const ycol = (second ? y2 : y) + (long)h * 128 + lane16 * 8;
-  for (int t = t_begin + sub; t < t_end; t += QT1 / 16) {
-    const u32x4 v = *(const u32x4*)(xcol + (long)t * xs_t);
-    *(u32x2*)(ycol + (long)(t - t_off) * H * 128) = quantize8(v, premul, sc);
+  if (threadIdx.x == 0 && blockIdx.z == 0) (second ? scales2 : scales)[(long)(c - t_off / chunk_tokens) * H + h] = sc;
+  // this workgroup's slice of the rows
+  const int per = (t_end - t_begin + (int)gridDim.z - 1) / (int)gridDim.z;
+  const int s_begin = t_begin + (int)blockIdx.z * per, s_end = min(t_end, s_begin + per);
+  char* const ycol = (second ? y2 : y) + (long)h * 128 + lane16 * 8 - (long)t_off * H * 128;
+  t = s_begin + sub;
+  for (; t + (UN - 1) * QROWS < s_end; t += UN * QROWS) {
+    u32x4 v[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) v[u] = *(const u32x4*)(xcol + (long)(t + u * QROWS) * xs_t);
+#pragma unroll
+    for (int u = 0; u < UN; ++u) *(u32x2*)(ycol + (long)(t + u * QROWS) * H * 128) = quantize8(v[u], premul, sc);
   }
+  for (; t < s_end; t += QROWS)
+    *(u32x2*)(ycol + (long)t * H * 128) = quantize8(*(const u32x4*)(xcol + (long)t * xs_t), premul, sc);
 }
 
 }  // namespace
@@ -610,16 +632,20 @@ hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream) {
 
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
                                int chunk_tokens, float premul, int pow2_scales, int n_first, char* y2, float* scales2,
-                               hipStream_t stream) {
+                               bool one_launch, hipStream_t stream) {
   const int n_chunks = (T + chunk_tokens - 1) / chunk_tokens;
   const int n = n_chunks * H;
   if (n <= 0) return hipSuccess;
-  // One launch when a group fits one workgroup's two passes and there are enough groups to spread over the chip
-  // (or a second destination, which only that kernel serves); both paths give the same bytes.
-  const bool one_launch = n_first < T || (min(chunk_tokens, T) <= 8192 && (n >= 64 || (long)T * H <= 65536));
+  // Unless asked for, one launch only when a group is small enough for one workgroup's two passes and there are
+  // enough groups to spread over the chip (a second destination is served by that kernel alone); both paths give
+  // the same bytes.
+  if (n_first < T || (min(chunk_tokens, T) <= 8192 && (n >= 64 || (long)T * H <= 65536))) one_launch = true;
   if (one_launch) {
     if (n_chunks > 65535) return hipErrorInvalidValue;
-    hipLaunchKernelGGL(quantize_groups_kernel, dim3(H, n_chunks), dim3(QT1), 0, stream, x, x_stride_t, x_stride_h, y,
+    // workgroups per group: towards two per CU over the launch, each slice at least four passes long
+    int share = (512 + n - 1) / n;
+    share = max(1, min(share, min(16, min(chunk_tokens, T) / (4 * QROWS))));
+    hipLaunchKernelGGL(quantize_groups_kernel, dim3(H, n_chunks, share), dim3(QT1), 0, stream, x, x_stride_t, x_stride_h, y,
                        scales, T, H, chunk_tokens, premul, pow2_scales, n_first, y2, scales2);
     return hipGetLastError();
   }

@@ -57,7 +57,8 @@ def test_one_launch_quantiser_with_two_destinations(dev):
     size above the one-launch limit of magi_quantize_fp8 gives the same bytes through either entry point."""
     g = torch.Generator().manual_seed(3)
     C, H, D = 48, 3, 128
-    for n_chunks, keep in ((5, 3), (4, 4), (3, 0), (1, 1)):
+    # (with few large groups several workgroups share a group: 1000-token chunks are cut in three uneven slices)
+    for n_chunks, keep, C in ((5, 3, 48), (4, 4, 48), (3, 0, 48), (1, 1, 48), (3, 1, 1000), (2, 2, 1111)):
         T = n_chunks * C
         big = (torch.randn(T, 2 * H * D, generator=g) * 3).bfloat16()
         x = big.view(T, H, 2 * D)[..., D:]  # the V half of an interleaved projection

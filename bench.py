@@ -275,20 +275,22 @@ def fp8_leg(inp, core_fl, bf16_tflops, steps, ref_rows, ref):
                 "frac": round(prep_bytes / (prep_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
         else:
             q8, qs = M.quantize_fp8(inp["q"], L, premul=1.0 / Q_PREMUL)
-        kw = dict(q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L, out=out8, return_lse=False,
-                  fp8_pow2_prescaled=pow2)
-        M.range_attention(q8, k8, v8, inp["q_ranges"], inp["k_ranges"], L, **kw)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(steps):
+        for fast in ((False, True) if pow2 else (False,)):  # the fast exp2 variant runs on the same operands
+            kw = dict(q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L, out=out8, return_lse=False,
+                      fp8_pow2_prescaled=pow2, fp8_fast_exp2=fast)
             M.range_attention(q8, k8, v8, inp["q_ranges"], inp["k_ranges"], L, **kw)
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1) / steps
-        tf = core_fl / (ms * 1e-3) / 1e12
-        res[mode] = {"achieved": round(tf, 2), "frac": round(tf / PEAK_FP8_TFLOPS, 4), "ms": round(ms, 3),
-                     "speedup_vs_bf16": round(tf / bf16_tflops, 3), "vs_fp32": deviation(out8[ref_rows], ref)}
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(steps):
+                M.range_attention(q8, k8, v8, inp["q_ranges"], inp["k_ranges"], L, **kw)
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / steps
+            tf = core_fl / (ms * 1e-3) / 1e12
+            res[mode + ("_fast_exp2" if fast else "")] = {
+                "achieved": round(tf, 2), "frac": round(tf / PEAK_FP8_TFLOPS, 4), "ms": round(ms, 3),
+                "speedup_vs_bf16": round(tf / bf16_tflops, 3), "vs_fp32": deviation(out8[ref_rows], ref)}
         del q8, k8, v8
     res["mode_of_the_layer_module"] = "pow2_prescaled"
     res["achieved"], res["frac"], res["ms"], res["speedup_vs_bf16"] = (res["pow2_prescaled"][k_] for k_ in

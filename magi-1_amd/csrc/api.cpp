@@ -91,6 +91,8 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     return fail(MAGI_ENOSYS, "magi_attn_fwd: k / v token strides above 2^23 elements are not implemented");
   if (p->dtype == MAGI_DTYPE_FP8_E4M3 && (p->flags & MAGI_ATTN_Q_PRESCALED))
     return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_Q_PRESCALED is a bf16 flag (fp8: MAGI_ATTN_FP8_POW2_PRESCALED)");
+  if ((p->flags & MAGI_ATTN_FP8_FAST_EXP2) && !(p->dtype == MAGI_DTYPE_FP8_E4M3 && (p->flags & MAGI_ATTN_FP8_POW2_PRESCALED)))
+    return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_FP8_FAST_EXP2 goes with fp8 and MAGI_ATTN_FP8_POW2_PRESCALED");
   if (p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_FP8_POW2_PRESCALED))
     return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_FP8_POW2_PRESCALED is an fp8 flag");
   if (!(p->score_bound >= 0.f)) return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound must be >= 0");

@@ -57,7 +57,9 @@ __device__ __forceinline__ void load_range(const int* r, int mode, int i, int to
   e = max(s, min(e, total));
 }
 
-template <bool POW2>
+// FASTP (with POW2): the probabilities come from a piecewise-linear exp2 built on the matrix pipe's scaling
+// instead of the quarter-rate v_exp_f32 (see the softmax below).
+template <bool POW2, bool FASTP = false>
 __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKernArgs a) {
   // Two (K tile, V tile) buffers as four separate objects that are only ever indexed statically: the compiler
   // then knows that a read of one buffer cannot alias the direct-to-LDS loads in flight to the other and does
@@ -231,9 +233,16 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   // row's maximum; there m starts at 0 and the first tile sets it.
   float m_run = POW2 ? 0.f : -__builtin_inff();
   float l_run = 0.f;
+  // FASTP: the score MFMAs carry 23 more on their scale exponent and accumulate onto (127 + shift - m) * 2^23, so a
+  // register holds (e + 127) * 2^23 for the exponent e of its probability: truncated to an integer that is the bit
+  // pattern of the fp32 number 2^floor(e) * (1 + frac(e)), exp2 with a linear mantissa (at most 6.2 % above 2^e,
+  // 4 % on average; the row sum is taken from the same values, so the average cancels and a relative spread of
+  // 2 % is what remains, beside the 2.7 % of the rounding to e4m3).  One full-rate conversion per score.
+  constexpr float XS = FASTP ? 8388608.f : 1.f;       // units of the accumulator per exponent unit
+  constexpr float XB = FASTP ? 127.f * 8388608.f : 0.f;  // accumulator value of exponent 0
   f32x16 neg_m;
 #pragma unroll
-  for (int v = 0; v < 16; ++v) neg_m[v] = 0.f;
+  for (int v = 0; v < 16; ++v) neg_m[v] = XB;
   float cur_shift = 0.f;
   bool first = true;
   const int e_q = (__builtin_bit_cast(int, q_sc) >> 23) & 0xff;  // E8M0 code of the (power-of-two) query scale
@@ -276,7 +285,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         if constexpr (!POW2) c = c_q * k_sc;                             // per-lane score scale inside this piece
         shift = uni(P_SHIFT + __builtin_amdgcn_logf(v_sc) - log2_vmax);  // <= 8
         unshift = uni(__builtin_amdgcn_exp2f(-shift));
-        e_k = (__builtin_bit_cast(int, k_sc) >> 23) & 0xff;  // E8M0 code of a power-of-two key scale
+        e_k = ((__builtin_bit_cast(int, k_sc) >> 23) & 0xff) + (FASTP ? 23 : 0);  // E8M0 code of a power-of-two key scale
       }
 
       auto read_k = [&](int t, int kk) -> i32x8 {
@@ -303,14 +312,14 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       ka[1] = read_k(0, 1);
       if constexpr (POW2) {
         if (shift != cur_shift) {  // a new scale chunk (wave-uniform): re-base the accumulator offset
-          const float ds = shift - cur_shift;
+          const float ds = (shift - cur_shift) * XS;
 #pragma unroll
           for (int v = 0; v < 16; ++v) neg_m[v] += ds;
           cur_shift = shift;
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[0], qf[0], neg_m, 0, 0, 0, e_k, 0, e_q);
+          s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[0], qf[0], neg_m, 0, 0, 0, e_k, 0, e_q);  // (FASTP: e_k carries + 23)
           if (t == 0) ka[0] = read_k(1, 0);
           __builtin_amdgcn_sched_barrier(0);  // (keeps each operand read one MFMA ahead of its use, where it is written)
           s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[1], qf[1], s_acc[t], 0, 0, 0, e_k, 0, e_q);
@@ -339,6 +348,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
             if (key >= pe) s_acc[t][v] = -__builtin_inff();
           }
       }
+      float psum = 0.f, psum2 = 0.f;
       float mx = max3(s_acc[0][0], s_acc[0][1], s_acc[0][2]);
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -347,12 +357,12 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       mx = half_swap_max(mx);
       if constexpr (POW2) {
         // s_acc already holds exponent - m_run + shift; a value above `shift` is a new row maximum
-        const float over = mx - shift;
+        const float over = mx - (shift * XS + XB);
         const bool raise = first || over > 0.f;
         if (__builtin_amdgcn_ballot_w64(raise) != 0) {
           const float delta = raise ? over : 0.f;
-          const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta);  // nothing to rescale on the first tile
-          m_run += delta;
+          const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta * (1.f / XS));  // nothing to rescale on the first tile
+          m_run += delta * (1.f / XS);
           l_run *= alpha;
 #pragma unroll
           for (int v = 0; v < 16; ++v) neg_m[v] -= delta;
@@ -368,12 +378,24 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           }
         }
         first = false;
+        auto pexp = [](float x) -> float {
+          if constexpr (FASTP) {  // (the conversion saturates at 0 for negative values and -inf: a probability of 0)
+            float r;
+            asm("v_cvt_u32_f32 %0, %1" : "=v"(r) : "v"(x));
+            return r;
+          } else
+            return __builtin_amdgcn_exp2f(x);
+        };
 #pragma unroll
         for (int n = 0; n < 8; ++n) {  // dword n = slots 4n .. 4n+3 = s_acc[n >> 2][4 (n & 3) .. +3]
-          const float p0 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 0]);
-          const float p1 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 1]);
-          const float p2 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 2]);
-          const float p3 = __builtin_amdgcn_exp2f(s_acc[n >> 2][4 * (n & 3) + 3]);
+          const float p0 = pexp(s_acc[n >> 2][4 * (n & 3) + 0]);
+          const float p1 = pexp(s_acc[n >> 2][4 * (n & 3) + 1]);
+          const float p2 = pexp(s_acc[n >> 2][4 * (n & 3) + 2]);
+          const float p3 = pexp(s_acc[n >> 2][4 * (n & 3) + 3]);
+          if constexpr (FASTP) {  // row sum by vector additions (see the row-sum MFMA below)
+            psum += p0 + p1;
+            psum2 += p2 + p3;
+          }
           // v_cvt_pk_fp8_f32 keeps the other half of its destination: start from p0's register (its high half is
           // overwritten by the second conversion) instead of a zeroed one
           int u = __builtin_bit_cast(int, p0);
@@ -415,11 +437,15 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       // exponentials alone take as long as its 8 MFMAs), not by the matrix pipe.  Every row of the product is the
       // sum over all 64 keys of the probabilities AS ROUNDED to e4m3, i.e. of exactly what the PV product uses, and
       // both lanes of a query get the full sum.  Issued ahead of the PV MFMAs and read after them.
+      // With FASTP the vector pipe has room again (one full-rate conversion per score instead of a quarter-rate
+      // exponential), so the row sum goes back to it (32 additions per lane of the values ahead of their rounding
+      // to e4m3, whose rounding errors average out over a row) and the matrix pipe keeps to its 8 MFMAs.
       __builtin_amdgcn_sched_barrier(0);
       i32x8 ones;
 #pragma unroll
       for (int n = 0; n < 8; ++n) ones[n] = n < 4 ? 0x22222222 : 0;  // fp4 e2m1 1.0 = 0b0010
-      const f32x16 rowsum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, zero16, 4, 0, 0, 0, 0, 0);
+      f32x16 rowsum = zero16;
+      if constexpr (!FASTP) rowsum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, zero16, 4, 0, 0, 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) {  // two V operands in flight, in alternating registers
@@ -427,7 +453,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         if (mb + 2 < 4) va[mb & 1] = read_v(mb + 2);
       }
       __builtin_amdgcn_sched_barrier(0);
-      l_run += rowsum[0] * unshift;
+      l_run += (FASTP ? psum + psum2 : rowsum[0]) * unshift;
     }
     k0 = k1;
     pe = pe1;
@@ -442,7 +468,9 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   }
 
   if (!wave_on) return;
-  const float l_tot = l_run;  // (the row-sum MFMA hands every lane the sum over all keys of its query)
+  // (the row-sum MFMA hands every lane the sum over all keys of its query; the vector sums of FASTP cover the keys
+  // of the lane's own half wave)
+  const float l_tot = FASTP ? l_run + __shfl_xor(l_run, 32) : l_run;
   const float inv = v_max * __builtin_amdgcn_exp2f(-P_SHIFT) / l_tot;
   // A lane holds four consecutive features per (mb, b), its partner in the other half wave the next four: the
   // halves trade the odd-b registers of the lower half for the even-b registers of the upper one, after which
@@ -623,7 +651,9 @@ __global__ __launch_bounds__(QT1) void quantize_groups_kernel(const char* x, lon
 
 hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-  if (a.flags & 1)
+  if ((a.flags & 1) && (a.flags & 4))
+    hipLaunchKernelGGL((attn_fwd_fp8_kernel<true, true>), dim3(grid), dim3(64 * NW), 0, stream, a);
+  else if (a.flags & 1)
     hipLaunchKernelGGL(attn_fwd_fp8_kernel<true>, dim3(grid), dim3(64 * NW), 0, stream, a);
   else
     hipLaunchKernelGGL(attn_fwd_fp8_kernel<false>, dim3(grid), dim3(64 * NW), 0, stream, a);

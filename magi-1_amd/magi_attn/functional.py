@@ -69,6 +69,7 @@ def range_attention(
     v2_scale: Optional[torch.Tensor] = None,
     scale_chunk_tokens: int = 0,
     fp8_pow2_prescaled: bool = False,
+    fp8_fast_exp2: bool = False,
     q_prescaled: bool = False,
     score_bound: float = 0.0,
     q_tile_rows: int = 0,
@@ -84,6 +85,8 @@ def range_attention(
 
     k2_scale / v2_scale (fp8, with k2 / v2): the side segment's scale rows in tables of their own, row 0 = the chunk
     that starts at k_split; without them k_scale / v_scale are indexed across k_split as one table.
+
+    fp8_fast_exp2 (with fp8_pow2_prescaled): piecewise-linear exp2 for the probabilities, MAGI_ATTN_FP8_FAST_EXP2.
 
     q_prescaled (bf16): q already carries softmax_scale * log2(e) (qk_prologue(..., q_premul=that)), so q . k is the
     exp2 exponent: the kernel skips its per-score multiply; softmax_scale is ignored.
@@ -152,7 +155,8 @@ def range_attention(
     a.dtype = _dtype_code(q)
     a.scale_chunk_tokens = int(scale_chunk_tokens)
     a.softmax_scale = 0.0 if softmax_scale is None else float(softmax_scale)
-    a.flags = (L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0) | (L.MAGI_ATTN_Q_PRESCALED if q_prescaled else 0)
+    a.flags = ((L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0) | (L.MAGI_ATTN_Q_PRESCALED if q_prescaled else 0)
+               | (L.MAGI_ATTN_FP8_FAST_EXP2 if fp8_fast_exp2 else 0))
     a.score_bound = float(score_bound)
     a.q_tile_rows = int(q_tile_rows)
     keep = None

@@ -148,9 +148,15 @@ def test_fp8_attention_parity(dev, L, dn, sp, Hq, Hkv, C):
 
 @pytest.mark.parametrize("L,dn,sp,Hq,Hkv,C", [(128, 1, 0, 1, 1, 128), (200, 3, 1, 6, 2, 200), (77, 2, 2, 3, 1, 50),
                                               (1536, 3, 0, 24, 8, 1536)])
-def test_fp8_pow2_prescaled_mode(dev, L, dn, sp, Hq, Hkv, C):
+@pytest.mark.parametrize("fast_exp2", [False, True])
+def test_fp8_pow2_prescaled_mode(dev, L, dn, sp, Hq, Hkv, C, fast_exp2):
     """Fast mode: power-of-two scales on the MFMA block-scale operands, softmax_scale * log2(e) folded into q at
-    quantisation.  Quantiser bit-exact with the oracle's; attention within the same stated tolerance."""
+    quantisation.  Quantiser bit-exact with the oracle's; attention within the same stated tolerance.
+    fast_exp2 (MAGI_ATTN_FP8_FAST_EXP2): probabilities 2^floor(e) (1 + frac(e)), up to 6.2 % above 2^e and 4 % on
+    average, normalised by their own sum: against the oracle on the original inputs the same bar holds; against
+    the oracle on the dequantised inputs, which isolates the kernel's own error, cosine >= 0.999 instead of 0.9995
+    (a 2 % spread of the weights beside the 2.7 % of their rounding to e4m3), and lse may sit up to
+    ln(1.062) = 0.06 above the exact one."""
     import math
 
     cs = 128 ** -0.5 * math.log2(math.e)
@@ -164,7 +170,7 @@ def test_fp8_pow2_prescaled_mode(dev, L, dn, sp, Hq, Hkv, C):
     assert torch.all(torch.frexp(ks.cpu())[0] == 0.5) and torch.all(torch.frexp(qs.cpu())[0] == 0.5)  # powers of two
     tq, tk = torch.tensor(qr, device=dev), torch.tensor(kr, device=dev)
     out, lse = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=C,
-                                 fp8_pow2_prescaled=True)
+                                 fp8_pow2_prescaled=True, fp8_fast_exp2=fast_exp2)
     err, cos = _per_head(out, O.range_attention(q, k, v, qr, kr))
     assert err <= 2 ** -5 * v.float().abs().max().item() and cos >= 0.998, (err, cos)
     # dequantised inputs (q side carries the folded scale, so the oracle runs with scale 1 in base 2)
@@ -172,17 +178,23 @@ def test_fp8_pow2_prescaled_mode(dev, L, dn, sp, Hq, Hkv, C):
     kd = O.dequantize_per_head_chunk(k8.cpu(), ks.cpu(), C)
     vd = O.dequantize_per_head_chunk(v8.cpu(), vs.cpu(), C)
     err, cos = _per_head(out, O.range_attention(qd, kd, vd, qr, kr, softmax_scale=1.0))
-    assert err <= 4e-2 and cos >= 0.9995, (err, cos)
+    assert err <= 4e-2 and cos >= (0.999 if fast_exp2 else 0.9995), (err, cos)
     lse_ref = O.range_attention_lse(qd, kd, vd, qr, kr, softmax_scale=1.0)
-    assert (lse.cpu() - lse_ref).abs().max() < 2e-2  # (sum of the e4m3-rounded probabilities, see above)
+    d_lse = lse.cpu() - lse_ref
+    if fast_exp2:
+        assert d_lse.min() > -2e-2 and d_lse.max() < 0.062 + 2e-2
+    else:
+        assert d_lse.abs().max() < 2e-2  # (sum of the e4m3-rounded probabilities, see above)
 
 
-@pytest.mark.parametrize("pow2", [False, True])
+@pytest.mark.parametrize("pow2", [False, True, "fast_exp2"])
 def test_fp8_scores_far_below_zero_from_the_first_tile(dev, pow2):
     """All scores near -260 in base-2 units (q and k anti-parallel): the running maximum starts far below its
     initial value, and the first tile's rescale factor 2^(+260) must not reach the (empty) accumulators."""
     import math
 
+    fast = pow2 == "fast_exp2"
+    pow2 = bool(pow2)
     g = torch.Generator().manual_seed(77)
     T, Hq, Hkv, D = 200, 2, 1, 128
     sign = torch.where(torch.rand(D, generator=g) < 0.5, -1.0, 1.0)
@@ -198,7 +210,7 @@ def test_fp8_scores_far_below_zero_from_the_first_tile(dev, pow2):
     tq = torch.tensor(qr, dtype=torch.int32, device=dev)
     tk = torch.tensor(kr, dtype=torch.int32, device=dev)
     out, lse = M.range_attention(q8, k8, v8, tq, tk, T, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=T,
-                                 fp8_pow2_prescaled=pow2)
+                                 fp8_pow2_prescaled=pow2, fp8_fast_exp2=fast)
     assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
     qd = O.dequantize_per_head_chunk(q8.cpu(), qs.cpu(), T)
     kd = O.dequantize_per_head_chunk(k8.cpu(), ks.cpu(), T)
@@ -246,7 +258,7 @@ def test_fp8_uneven_scales_and_two_segments(dev):
     assert (out2.float() - out.float()).abs().max().item() <= 4e-2 * deq.abs().max().item()
 
 
-@pytest.mark.parametrize("mode", ["generic", "pow2_prescaled"])
+@pytest.mark.parametrize("mode", ["generic", "pow2_prescaled", "pow2_prescaled_fast_exp2"])
 def test_fp8_full_size_720p_accuracy(dev, mode):
     """Benchmark shape in fp8, in both scale modes: sampled-row accuracy against fp32 math on the original tensors.
     pow2_prescaled is the mode the layer module and the benchmark run (power-of-two scales on the MFMA's block-scale
@@ -263,14 +275,14 @@ def test_fp8_full_size_720p_accuracy(dev, mode):
     k = torch.randn((sp + dn) * L, Hkv, D, device=dev, generator=g)
     k = (k * torch.rsqrt(k.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
     v = torch.randn((sp + dn) * L, Hkv, D, device=dev, generator=g).bfloat16()
-    pow2 = mode == "pow2_prescaled"
+    pow2 = mode != "generic"
     q8, qs = M.quantize_fp8(q, L, premul=D ** -0.5 * math.log2(math.e) if pow2 else 1.0, pow2_scales=pow2)
     k8, ks = M.quantize_fp8(k, L, pow2_scales=pow2)
     v8, vs = M.quantize_fp8(v, L, pow2_scales=pow2)
     qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
     tq, tk = torch.tensor(qr, device=dev), torch.tensor(kr, device=dev)
     out, _ = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L,
-                               return_lse=False, fp8_pow2_prescaled=pow2)
+                               return_lse=False, fp8_pow2_prescaled=pow2, fp8_fast_exp2=mode.endswith("fast_exp2"))
     torch.cuda.synchronize()
     G = Hq // Hkv
     rs = np.random.default_rng(0)
@@ -327,7 +339,9 @@ def test_fp8_randomised_ranges_chunks_and_splits(dev):
         v8, vsc = M.quantize_fp8(v.to(dev), C, pow2_scales=pow2)
         tq = torch.tensor(qr, dtype=torch.int32, device=dev)
         tk = torch.tensor(kr, dtype=torch.int32, device=dev)
-        kw = dict(q_scale=qs, k_scale=ksc, v_scale=vsc, scale_chunk_tokens=C, fp8_pow2_prescaled=pow2, return_lse=False)
+        fast = pow2 and case % 4 == 3  # every other power-of-two case with the piecewise-linear exp2
+        kw = dict(q_scale=qs, k_scale=ksc, v_scale=vsc, scale_chunk_tokens=C, fp8_pow2_prescaled=pow2, return_lse=False,
+                  fp8_fast_exp2=fast)
         k1, v1 = k8, v8
         if case % 3 == 2:
             split = int(rng.integers(0, Tk + 1))
@@ -343,7 +357,8 @@ def test_fp8_randomised_ranges_chunks_and_splits(dev):
         rel = ((out.double().cpu() - ref.double()).abs().max() / ref.abs().max().clamp_min(1e-6)).item()
         # P is rounded to e4m3 (relative error <= 2^-4 per weight); with few keys nothing averages out, so the bound
         # relative to max|ref| is 2^-4 (MAGI_TEST_SWEEP_CASES=400 stays below it; case 88 reaches 4.2e-2)
-        assert rel <= 2 ** -4, f"case {case}: {rel}"
+        # (fast exp2: each weight up to 6.2 % high before the normalisation on top of that)
+        assert rel <= (0.1 if fast else 2 ** -4), f"case {case}: {rel}"
 
 
 def test_fp8_many_segments_with_empty_ones(dev):

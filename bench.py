@@ -292,8 +292,8 @@ def fp8_leg(inp, core_fl, bf16_tflops, steps, ref_rows, ref):
                 "achieved": round(tf, 2), "frac": round(tf / PEAK_FP8_TFLOPS, 4), "ms": round(ms, 3),
                 "speedup_vs_bf16": round(tf / bf16_tflops, 3), "vs_fp32": deviation(out8[ref_rows], ref)}
         del q8, k8, v8
-    res["mode_of_the_layer_module"] = "pow2_prescaled"
-    res["achieved"], res["frac"], res["ms"], res["speedup_vs_bf16"] = (res["pow2_prescaled"][k_] for k_ in
+    res["mode_of_the_layer_module"] = "pow2_prescaled_fast_exp2"
+    res["achieved"], res["frac"], res["ms"], res["speedup_vs_bf16"] = (res["pow2_prescaled_fast_exp2"][k_] for k_ in
                                                                        ("achieved", "frac", "ms", "speedup_vs_bf16"))
     return res
 

@@ -170,16 +170,19 @@ class FullyParallelAttention(torch.nn.Module):
     def __init__(self, hidden_size: int, num_attention_heads: int, num_query_groups: int, kv_channels: int = 128,
                  layer_number: int = 0, layernorm_epsilon: float = 1e-6, apply_layernorm_1p: bool = True,
                  xattn_cond_hidden_ratio: float = 1.0, params_dtype=torch.bfloat16, device=None,
-                 attention_dtype: str = "bf16"):
+                 attention_dtype: str = "bf16", fp8_fast_exp2: bool = True):
         """attention_dtype "fp8" (not in the reference, which has no fp8 attention) runs the self-attention on
         e4m3 operands with per-(video chunk, head) power-of-two scales and keeps the KV cache in that form
-        (Fp8KVCache); the cross attention and everything else stay in bf16."""
+        (Fp8KVCache); the cross attention and everything else stay in bf16.
+        fp8_fast_exp2: the fp8 kernel's piecewise-linear exp2 (MAGI_ATTN_FP8_FAST_EXP2: about 10 % faster, the
+        output within the same accuracy bar as with the exact exponential); False for the exact one."""
         super().__init__()
         if kv_channels != 128:
             raise NotImplementedError("head_dim 128 only")
         if attention_dtype not in ("bf16", "fp8"):
             raise ValueError("attention_dtype must be 'bf16' or 'fp8'")
         self.attention_dtype = attention_dtype
+        self.fp8_fast_exp2 = bool(fp8_fast_exp2)
         # forward() has the prologue fold softmax_scale * log2(e) into q ahead of q's one rounding to bf16 and tells
         # the attention kernel so (no per-score multiply there); get_q / get_qkv return q unscaled, as the reference
         self._q_premul = kv_channels ** -0.5 * math.log2(math.e)
@@ -299,7 +302,7 @@ class FullyParallelAttention(torch.nn.Module):
         gk, bk = self.k_layernorm.gamma_beta_fp32()
         pro = dict(Hq=Hq, Hkv=Hkv, q_scale=qs_c, k_scale=ks_c, eps=self.eps, q_premul=self._q_premul)
         kw = dict(q_scale=self._const_scale_table(qs_c, n_chunks, Hq, dev), scale_chunk_tokens=Lc,
-                  fp8_pow2_prescaled=True, out=out, return_lse=False)
+                  fp8_pow2_prescaled=True, fp8_fast_exp2=self.fp8_fast_exp2, out=out, return_lse=False)
         f8 = torch.float8_e4m3fn
         if not use_cache:
             q8, k8, _ = qk_prologue_fp8(q_raw, k_raw, rope, gq, bq, gk, bk, **pro)

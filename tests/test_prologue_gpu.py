@@ -431,7 +431,8 @@ def test_layer_with_arena_backed_cache(dev):
     assert torch.isnan(arena.layer(2)).all() and torch.isnan(arena.layer(4)).all()  # other layers untouched
 
 
-def test_layer_with_fp8_self_attention_and_fp8_cache(dev):
+@pytest.mark.parametrize("fast_exp2", [True, False])
+def test_layer_with_fp8_self_attention_and_fp8_cache(dev, fast_exp2):
     """attention_dtype="fp8": same schedule as above through two layers with identical weights, one bf16 and one
     fp8.  The reference has no fp8 attention (parity unpinned by it); the bf16 layer, itself checked against the
     oracle above, is the yardstick: per step cosine >= 0.998 and max-abs <= 2^-5 max|V| on the self-attention
@@ -446,7 +447,8 @@ def test_layer_with_fp8_self_attention_and_fp8_cache(dev):
     n_chunks = 6
     ref_layer = _make_layer(dev, hidden, Hq, Hkv, seed=5)
     torch.manual_seed(5)
-    fp8_layer = MOD.FullyParallelAttention(hidden, Hq, Hkv, layer_number=3, device=dev, attention_dtype="fp8")
+    fp8_layer = MOD.FullyParallelAttention(hidden, Hq, Hkv, layer_number=3, device=dev, attention_dtype="fp8",
+                                           fp8_fast_exp2=fast_exp2)
     fp8_layer.load_state_dict(ref_layer.state_dict())
     rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
     ip_ref, ip_fp8 = P.InferenceParams(1, n_chunks * L), P.InferenceParams(1, n_chunks * L)

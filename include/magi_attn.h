@@ -223,6 +223,47 @@ typedef struct magi_prologue_args {
 int magi_qk_prologue(const magi_prologue_args* args, void* stream);
 
 /*
+ * The four projections of the attention layer and the prologue in one launch: a bf16 GEMM
+ *     [S, K] x [N, K]^T,  N = (Hq + 2 Hkv + Hqx) * 128,  rows of w ordered  q heads | k heads | v heads | qx heads
+ * whose epilogue does to every (token, head) block of 128 columns what magi_qk_prologue does to the raw
+ * projections: round to bf16 (the projection's output dtype), per-head norm, partial rotary, q_premul, cast, and
+ * store q to q_out, k and v to the cache rows (kv_out / kv_tail as in magi_prologue_args), the cross-attention
+ * q projection UNNORMALISED to qx_out [S, Hqx, D] (magi_attn_fwd normalises it while loading, q_norm_*).
+ * Stands in for CustomLayerNormLinear's four linear layers after its LayerNorm
+ * (inference/model/dit/dit_module.py:390-425: forward_q / forward_qx / forward_k / forward_v on the output of
+ * forward_ln, called at :1153 and :954, 971, 986, 1007) followed by get_q / get_k / get_v (:953-996); the raw
+ * projections never reach memory.  fp32 accumulation, so a raw value may differ from a library GEMM's by one bf16
+ * rounding where the accumulation order decides it.
+ * x [S, K] bf16 (row stride in elements), w [N, K] bf16; K a multiple of 64; Hq + 2 Hkv + Hqx even;
+ * rope [S / batch, 96] fp32 (sin | cos) or NULL: this entry point implements rotary_dim 96 (R2 = 48) only.
+ */
+typedef struct magi_qkv_proj_args {
+  const void* x;
+  const void* w;
+  int64_t x_stride, w_stride;
+  int32_t S, K;
+  int32_t Hq, Hkv, Hqx, D;
+  const float* rope;
+  int32_t R2;
+  const float* gq;
+  const float* bq;
+  const float* gk;
+  const float* bk;
+  int32_t norm_kind;
+  float eps;
+  int32_t batch;
+  float q_premul;
+  void* q_out;
+  void* kv_out;
+  void* kv_tail;
+  int64_t kv_stride_t, kv_tail_stride_t;
+  int32_t n_cache_rows;
+  void* qx_out;
+} magi_qkv_proj_args;
+
+int magi_qkv_proj_prologue(const magi_qkv_proj_args* args, void* stream);
+
+/*
  * LayerNorm of the layer input over its last axis: x [rows, cols] bf16 -> y [rows, cols] bf16 with fp32
  * statistics, y = (x - mean) / sqrt(var + eps) * weight + bias (plain weight, not the "+1" form).
  * Stands in for torch.nn.LayerNorm in CustomLayerNormLinear.forward_ln (dit_module.py:401, 412-413;

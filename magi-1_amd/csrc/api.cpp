@@ -296,6 +296,73 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   return MAGI_OK;
 }
 
+int magi_qkv_proj_prologue(const magi_qkv_proj_args* p, void* stream) {
+  if (!p) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: args is NULL");
+  if (p->D != 128) return fail(MAGI_ENOSYS, "magi_qkv_proj_prologue: head_dim %d not implemented (128 only)", p->D);
+  if (p->S < 0 || p->K <= 0 || p->Hq < 0 || p->Hkv < 0 || p->Hqx < 0)
+    return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: bad size");
+  const int heads = p->Hq + 2 * p->Hkv + p->Hqx;
+  if (p->S == 0 || heads == 0) return MAGI_OK;
+  if (p->K % 64) return fail(MAGI_ENOSYS, "magi_qkv_proj_prologue: K=%d is not a multiple of 64", p->K);
+  if (heads % 2) return fail(MAGI_ENOSYS, "magi_qkv_proj_prologue: an odd number of heads (%d) is not implemented", heads);
+  if (p->rope && p->R2 != 48 && p->R2 != 0)
+    return fail(MAGI_ENOSYS, "magi_qkv_proj_prologue: R2=%d not implemented (48, or 0 / NULL rope for none)", p->R2);
+  if (p->norm_kind < 0 || p->norm_kind > 2) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: norm_kind %d", p->norm_kind);
+  if (p->batch < 0) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: negative batch");
+  if (!p->x || !p->w) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: NULL x / w");
+  if (p->x_stride < p->K || p->w_stride < p->K) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: row stride below K");
+  if (p->Hq > 0 && !p->q_out) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: NULL q_out");
+  if (p->Hqx > 0 && !p->qx_out) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: NULL qx_out");
+  if (p->n_cache_rows < 0 || p->n_cache_rows > p->S)
+    return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: n_cache_rows %d outside [0, S=%d]", p->n_cache_rows, p->S);
+  if (p->Hkv > 0 && p->n_cache_rows > 0 && !p->kv_out) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: NULL kv_out");
+  if (p->Hkv > 0 && p->n_cache_rows < p->S && !p->kv_tail)
+    return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: kv_tail needed for rows >= n_cache_rows");
+  if (p->norm_kind != MAGI_NORM_NONE && ((p->Hq > 0 && !p->gq) || (p->Hkv > 0 && !p->gk)))
+    return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: NULL gamma");
+  if (p->x_stride % 8 || p->w_stride % 8 || p->kv_stride_t % 8 || p->kv_tail_stride_t % 8)
+    return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: strides must keep rows 16-byte aligned");
+  if (!aligned16(p->x) || !aligned16(p->w) || !aligned16(p->q_out) || !aligned16(p->kv_out) || !aligned16(p->kv_tail) ||
+      !aligned16(p->qx_out) || !aligned16(p->rope) || !aligned16(p->gq) || !aligned16(p->bq) || !aligned16(p->gk) ||
+      !aligned16(p->bk))
+    return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: buffers must be 16-byte aligned");
+  // (the loader addresses a workgroup's 256 rows with 32-bit byte offsets)
+  if (p->x_stride > (1 << 21) || p->w_stride > (1 << 21))
+    return fail(MAGI_ENOSYS, "magi_qkv_proj_prologue: row strides above 2^21 elements are not implemented");
+  if (!(p->q_premul == p->q_premul) || std::fabs(p->q_premul) > 1e30f)
+    return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: q_premul is not finite");
+  magi::QkvGemmKernArgs a;
+  std::memset(&a, 0, sizeof(a));
+  a.x = static_cast<const char*>(p->x);
+  a.w = static_cast<const char*>(p->w);
+  a.rope = (p->rope && p->R2 == 48) ? p->rope : nullptr;
+  a.gq = p->gq;
+  a.bq = p->bq;
+  a.gk = p->gk;
+  a.bk = p->bk;
+  a.q_out = static_cast<char*>(p->q_out);
+  a.kv_out = static_cast<char*>(p->kv_out);
+  a.kv_tail = static_cast<char*>(p->kv_tail);
+  a.qx_out = static_cast<char*>(p->qx_out);
+  a.x_stride = p->x_stride * 2;
+  a.w_stride = p->w_stride * 2;
+  a.kv_stride_t = p->kv_stride_t * 2;
+  a.kv_tail_stride_t = p->kv_tail_stride_t * 2;
+  a.S = p->S;
+  a.K = p->K;
+  a.n_cache_rows = p->n_cache_rows;
+  a.Hq = p->Hq;
+  a.Hkv = p->Hkv;
+  a.Hqx = p->Hqx;
+  a.norm_kind = p->norm_kind;
+  a.eps = p->eps;
+  a.batch = p->batch > 1 ? p->batch : 1;
+  a.q_premul = p->q_premul == 0.f ? 1.f : p->q_premul;
+  hipError_t e = magi::launch_qkv_gemm_prologue(a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "magi_qkv_proj_prologue launch");
+  return MAGI_OK;
+}
+
 int magi_layer_norm(const void* x, int64_t x_stride, const void* weight, const void* bias, int32_t params_fp32,
                     void* y, int64_t y_stride, int64_t rows, int32_t cols, float eps, void* stream) {
   if (rows < 0 || cols < 0) return fail(MAGI_EINVAL, "magi_layer_norm: negative size");

@@ -74,6 +74,31 @@ struct PrologueKernArgs {
 };
 hipError_t launch_prologue(const PrologueKernArgs& a, hipStream_t stream);
 
+// The four projections as one GEMM with the prologue as its epilogue.  Strides in BYTES.
+struct QkvGemmKernArgs {
+  const char* x;  // [S, K] bf16
+  const char* w;  // [(Hq + 2 Hkv + Hqx) * 128, K] bf16, rows ordered q | k | v | qx heads
+  const float* rope;
+  const float* gq;
+  const float* bq;
+  const float* gk;
+  const float* bk;
+  char* q_out;
+  char* kv_out;
+  char* kv_tail;
+  char* qx_out;
+  long x_stride, w_stride;
+  long kv_stride_t, kv_tail_stride_t;
+  int S, K, n_cache_rows;
+  int Hq, Hkv, Hqx;
+  int norm_kind;
+  float eps;
+  int batch;
+  float q_premul;
+  int n_row_tiles, n_col_tiles;  // filled by the launcher
+};
+hipError_t launch_qkv_gemm_prologue(const QkvGemmKernArgs& a, hipStream_t stream);
+
 hipError_t launch_head_norm(const char* x, long x_stride_t, long x_stride_h, const float* gamma, const float* beta,
                             char* y, int S, int H, int norm_kind, float eps, hipStream_t stream);
 hipError_t launch_layer_norm(const char* x, long x_stride, const void* w, const void* b, int params_fp32, char* y,

@@ -66,6 +66,20 @@ class PrologueArgs(C.Structure):
     ]
 
 
+class QkvProjArgs(C.Structure):
+    _fields_ = [
+        ("x", C.c_void_p), ("w", C.c_void_p), ("x_stride", C.c_int64), ("w_stride", C.c_int64),
+        ("S", C.c_int32), ("K", C.c_int32),
+        ("Hq", C.c_int32), ("Hkv", C.c_int32), ("Hqx", C.c_int32), ("D", C.c_int32),
+        ("rope", C.c_void_p), ("R2", C.c_int32),
+        ("gq", C.c_void_p), ("bq", C.c_void_p), ("gk", C.c_void_p), ("bk", C.c_void_p),
+        ("norm_kind", C.c_int32), ("eps", C.c_float), ("batch", C.c_int32), ("q_premul", C.c_float),
+        ("q_out", C.c_void_p), ("kv_out", C.c_void_p), ("kv_tail", C.c_void_p),
+        ("kv_stride_t", C.c_int64), ("kv_tail_stride_t", C.c_int64), ("n_cache_rows", C.c_int32),
+        ("qx_out", C.c_void_p),
+    ]
+
+
 class QuantizeArgs(C.Structure):
     _fields_ = [
         ("x", C.c_void_p), ("x_stride_t", C.c_int64), ("x_stride_h", C.c_int64),
@@ -77,7 +91,7 @@ class QuantizeArgs(C.Structure):
 
 
 EXPORTS = ("magi_version", "magi_last_error", "magi_attn_fwd", "magi_qk_prologue", "magi_head_norm",
-           "magi_apply_rotary", "magi_quantize_fp8", "magi_quantize_fp8_split", "magi_layer_norm")
+           "magi_apply_rotary", "magi_quantize_fp8", "magi_quantize_fp8_split", "magi_layer_norm", "magi_qkv_proj_prologue")
 
 _lib = None
 
@@ -109,6 +123,8 @@ def lib() -> C.CDLL:
         l.magi_quantize_fp8.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32,
                                         C.c_int32, C.c_int32, C.c_int32, C.c_float, C.c_int32, C.c_void_p]
         l.magi_quantize_fp8.restype = C.c_int
+        l.magi_qkv_proj_prologue.argtypes = [C.POINTER(QkvProjArgs), C.c_void_p]
+        l.magi_qkv_proj_prologue.restype = C.c_int
         l.magi_quantize_fp8_split.argtypes = [C.POINTER(QuantizeArgs), C.c_void_p]
         l.magi_quantize_fp8_split.restype = C.c_int
         _lib = l

@@ -344,6 +344,67 @@ def qk_prologue_fp8(q_raw, k_raw, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int, q_
     return q_out, k_out, k_tail
 
 
+def qkv_proj_prologue(x: torch.Tensor, w: torch.Tensor, rope, gq, bq, gk, bk, *, Hq: int, Hkv: int, Hqx: int = 0,
+                      eps: float = 1e-6, norm_kind: int = L.MAGI_NORM_LAYERNORM_1P, kv_out: Optional[torch.Tensor] = None,
+                      n_cache_rows: Optional[int] = None, kv_tail: Optional[torch.Tensor] = None,
+                      q_out: Optional[torch.Tensor] = None, qx_out: Optional[torch.Tensor] = None, batch: int = 1,
+                      q_premul: float = 1.0):
+    """The four projections and the prologue in one launch (magi_qkv_proj_prologue): x [S, K] bf16 (the normalised
+    hidden states), w [(Hq + 2 Hkv + Hqx) * 128, K] bf16 with rows ordered q | k | v | qx heads.  Destinations as in
+    qk_prologue; qx_out [S, Hqx, 128] receives the cross-attention q projection unnormalised.
+    Returns (q [S, Hq, 128], kv_out, kv_tail, qx_out)."""
+    D = 128
+    if x.dim() != 2 or w.dim() != 2 or x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        raise ValueError("x and w must be 2-D bf16 tensors")
+    if x.stride(1) != 1 or w.stride(1) != 1 or x.shape[1] != w.shape[1] or w.shape[0] != (Hq + 2 * Hkv + Hqx) * D:
+        raise ValueError("x [S, K] and w [(Hq + 2 Hkv + Hqx) * 128, K] must have contiguous rows of the same length")
+    if not x.is_cuda or w.device != x.device:
+        raise ValueError("x and w must live on the same device (there is no CPU path)")
+    S, K = x.shape
+    dev = x.device
+    if q_out is None:
+        q_out = torch.empty((S, Hq, D), dtype=torch.bfloat16, device=dev)
+    if qx_out is None and Hqx:
+        qx_out = torch.empty((S, Hqx, D), dtype=torch.bfloat16, device=dev)
+    if kv_out is None and kv_tail is None:
+        kv_out = torch.empty((S, Hkv, 2 * D), dtype=torch.bfloat16, device=dev)
+        n_cache_rows = S
+    if n_cache_rows is None:
+        n_cache_rows = S if kv_tail is None else 0
+    for name, t, H in (("q_out", q_out, Hq), ("qx_out", qx_out, Hqx)):
+        if t is not None and (t.dtype != torch.bfloat16 or tuple(t.shape) != (S, H, D) or not t.is_contiguous()):
+            raise ValueError(f"{name} must be a contiguous bf16 [S, heads, 128] tensor")
+    for name, t in (("kv_out", kv_out), ("kv_tail", kv_tail)):
+        if t is not None and (t.dtype != torch.bfloat16 or t.dim() != 3 or t.shape[1:] != (Hkv, 2 * D)
+                              or t.stride(2) != 1 or t.stride(1) != 2 * D):
+            raise ValueError(f"{name} must be bf16 [rows, Hkv, 2*D] with contiguous heads")
+    if kv_out is not None and kv_out.shape[0] < n_cache_rows:
+        raise ValueError("kv_out is shorter than n_cache_rows")
+    if kv_tail is not None and kv_tail.shape[0] < S - n_cache_rows:
+        raise ValueError("kv_tail is shorter than S - n_cache_rows")
+    f32 = lambda t: None if t is None else t.to(torch.float32).contiguous()
+    gq, bq, gk, bk = f32(gq), f32(bq), f32(gk), f32(bk)
+    a = L.QkvProjArgs()
+    R2 = 0
+    if rope is not None:
+        if rope.dtype != torch.float32 or rope.dim() != 2 or rope.shape[0] * max(batch, 1) != S or not rope.is_contiguous():
+            raise ValueError("rope must be a contiguous fp32 [S / batch, 2*R2] tensor")
+        R2 = rope.shape[1] // 2
+    a.x, a.w, a.x_stride, a.w_stride = _ptr(x), _ptr(w), x.stride(0), w.stride(0)
+    a.S, a.K = S, K
+    a.Hq, a.Hkv, a.Hqx, a.D = Hq, Hkv, Hqx, D
+    a.rope, a.R2 = _ptr(rope), R2
+    a.gq, a.bq, a.gk, a.bk = _ptr(gq), _ptr(bq), _ptr(gk), _ptr(bk)
+    a.norm_kind, a.eps, a.batch, a.q_premul = int(norm_kind), float(eps), int(batch), float(q_premul)
+    a.q_out, a.kv_out, a.kv_tail, a.qx_out = _ptr(q_out), _ptr(kv_out), _ptr(kv_tail), _ptr(qx_out)
+    a.kv_stride_t = 0 if kv_out is None else kv_out.stride(0)
+    a.kv_tail_stride_t = 0 if kv_tail is None else kv_tail.stride(0)
+    a.n_cache_rows = int(n_cache_rows)
+    with torch.cuda.device(dev):
+        L.check(L.lib().magi_qkv_proj_prologue(C.byref(a), _stream()))
+    return q_out, kv_out, kv_tail, qx_out
+
+
 def pow2_scale_for(bound: float) -> float:
     """Smallest power of two s with bound / s <= 448 (the largest e4m3 value): the scale to quantise values of
     magnitude <= bound with.  e4m3 being a floating-point format, a bound that is a few times too large costs

@@ -96,6 +96,7 @@ struct QkvGemmKernArgs {
   int batch;
   float q_premul;
   int n_row_tiles, n_col_tiles;  // filled by the launcher
+  int variant;                   // 4: the 4-wavefront form (tuning builds)
 };
 hipError_t launch_qkv_gemm_prologue(const QkvGemmKernArgs& a, hipStream_t stream);
 

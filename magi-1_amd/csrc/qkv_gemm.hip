@@ -16,8 +16,13 @@
 // operand, tokens as the B operand): a lane then holds ONE token per 32-token block and 64 of its 128 features
 // (its partner in the other half wave the other 64), which is the layout the epilogue wants: the norm statistics
 // need one exchange between the half waves, and a rotary pair (f, f + 48) lives in one lane.
-// Per 64-step a wave issues 24 operand reads of 16 bytes for 32 MFMAs.
+// Per 64-step a wave issues 24 operand reads of 16 bytes for 32 MFMAs: 0.75 KB of LDS reads per MFMA, 96 bytes per
+// clock and CU at the full MFMA rate, beside 32 for filling the slices.  The CU's LDS delivers about 157 bytes per
+// clock to ds_read_b128 (measured with a read-only loop), so LDS bandwidth is what bounds this kernel; the library
+// GEMM it competes with sits at the same wall with 128 x 128 per wavefront (0.5 KB per MFMA).
 #include "attn_common.h"
+
+#include <cstdlib>
 
 namespace magi {
 namespace {
@@ -27,16 +32,22 @@ constexpr int BNC = 256; // columns per workgroup (two heads)
 constexpr int BK = 64;   // k per step
 constexpr int ROWB = BK * 2;  // bytes per LDS row
 constexpr int TILE = BM * ROWB;  // 32 KB per matrix per stage
-constexpr int NWAVES = 8;
 constexpr int D = 128;
 constexpr int R2 = 48;  // rotary pairs (the MAGI-1 layout: rotary_dim 96 of 128)
 
-__global__ __launch_bounds__(64 * NWAVES, 1) void qkv_gemm_prologue_kernel(const QkvGemmKernArgs a) {
+// MB: blocks of 32 tokens per wavefront.  MB = 2 (shipped): 8 wavefronts (two per SIMD), 128 accumulator registers
+// each.  MB = 4: 4 wavefronts (one per SIMD) with 256 accumulator registers each, 0.5 instead of 0.75 KB of LDS
+// operand reads per MFMA, but nothing to hide a wave's own waits behind; measured 2 % slower.
+template <int MB>
+__global__ __launch_bounds__(64 * (16 / MB), 1) void qkv_gemm_prologue_kernel(const QkvGemmKernArgs a) {
+  constexpr int NWAVES = 16 / MB;
+  constexpr int LOADS = 32 / NWAVES;  // wave-loads (8 rows each) per wave per matrix per step
   extern __shared__ __attribute__((aligned(1024))) unsigned char smem[];
   unsigned char* const sX0 = smem;
   unsigned char* const sW0 = smem + TILE;
   unsigned char* const sX1 = smem + 2 * TILE;
   unsigned char* const sW1 = smem + 3 * TILE;
+  unsigned char* const sJunk = smem + 4 * TILE;  // 1 KB that nothing reads (destination of the cache-warming loads)
 
   // ---- which tile: blockIdx % 8 is the XCD; an XCD walks blocks of 8 token tiles x all column tiles, token tile
   // fastest, so that the ~32 workgroups it runs at a time share 8 X slices and 4 W slices through its L2 ----
@@ -54,7 +65,8 @@ __global__ __launch_bounds__(64 * NWAVES, 1) void qkv_gemm_prologue_kernel(const
   const int l = tid & 63, i = l & 31, g = l >> 5;
   const int wn = w & 1, wm = w >> 1;
 
-  // ---- loader: a wave-load of 64 x 16 bytes fills 8 LDS rows; wave w takes row groups w, w + 8, w + 16, w + 24
+  const int n_steps = a.K / BK;
+  // ---- loader: a wave-load of 64 x 16 bytes fills 8 LDS rows; wave w takes row groups w, w + NWAVES, ...
   // of both matrices.  Lane l sits at row (l >> 3) of its group, slot l & 7, and fetches the logical chunk that
   // belongs there under the swizzle.
   const int lr = l >> 3, sl = l & 7;
@@ -71,53 +83,93 @@ __global__ __launch_bounds__(64 * NWAVES, 1) void qkv_gemm_prologue_kernel(const
   auto issue = [&](int kstep, unsigned char* sX, unsigned char* sW) __attribute__((always_inline)) {
     const unsigned kb = (unsigned)kstep * (unsigned)ROWB;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, LDS_PTR(void, sX + (w + 8 * j) * 1024), 16, vx,
-                                               (int)(kb + (unsigned)(64 * j) * (unsigned)a.x_stride), 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, LDS_PTR(void, sW + (w + 8 * j) * 1024), 16, vw,
-                                               (int)(kb + (unsigned)(64 * j) * (unsigned)a.w_stride), 0, 0);
+    for (int j = 0; j < LOADS; ++j) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, LDS_PTR(void, sX + (w + NWAVES * j) * 1024), 16, vx,
+                                               (int)(kb + (unsigned)(8 * NWAVES * j) * (unsigned)a.x_stride), 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, LDS_PTR(void, sW + (w + NWAVES * j) * 1024), 16, vw,
+                                               (int)(kb + (unsigned)(8 * NWAVES * j) * (unsigned)a.w_stride), 0, 0);
+    }
+    // Warm the caches for the slice after that one: one 4-byte load per 128-byte row segment, issued BEHIND the
+    // loads above (loads complete in order, so the wait in front of the barrier can leave exactly these
+    // outstanding) into LDS that nothing reads.  A slice is requested by the ~32 workgroups of an XCD at about the
+    // same time and the first request goes to HBM (measured: 6 % on the 4-wavefront form, which has nothing to
+    // hide a wait behind; no difference on the 8-wavefront form).
+    const unsigned kt = (unsigned)min(kstep + 1, n_steps - 1) * (unsigned)ROWB;
+    if constexpr (MB == 4) {
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, LDS_PTR(void, sJunk), 4, (unsigned)tid * (unsigned)a.x_stride, (int)kt, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, LDS_PTR(void, sJunk + 256), 4, (unsigned)tid * (unsigned)a.w_stride, (int)kt, 0, 0);
+    } else {
+      if (w < 4)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, LDS_PTR(void, sJunk), 4, (unsigned)tid * (unsigned)a.x_stride, (int)kt, 0, 0);
+      else
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, LDS_PTR(void, sJunk + 256), 4, (unsigned)(tid - 256) * (unsigned)a.w_stride, (int)kt, 0, 0);
     }
   };
+  constexpr int TOUCHES = MB == 4 ? 2 : 1;  // cache-warming loads per wave per step
 
   // ---- operand reads: row 32 blk + i of a slice, 16-byte chunk (2 kk + g) ^ ((i >> 1) & 7) ----
   const int sw = ((g ^ ((i >> 1) & 7)) << 4);
   const int base_w = (128 * wn + i) * ROWB + sw;  // + nb * 32 rows
-  const int base_x = (64 * wm + i) * ROWB + sw;   // + mb * 32 rows
+  const int base_x = (32 * MB * wm + i) * ROWB + sw;   // + mb * 32 rows
 
-  f32x16 acc[4][2];  // [feature block of 32][token block of 32]
+  f32x16 acc[4][MB];  // [feature block of 32][token block of 32]
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[nb][mb][v] = 0.f;
 
-  const int n_steps = a.K / BK;
+  bf16x8 wf[2][4], xf[2][MB];  // two sets of operand fragments (one k block of 16 each)
+  auto fetch = [&](const unsigned char* X, const unsigned char* W, int kk, int s) __attribute__((always_inline)) {
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) wf[s][nb] = *LDS_PTR(const bf16x8, W + ((base_w ^ (kk << 5)) + nb * 32 * ROWB));
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xf[s][mb] = *LDS_PTR(const bf16x8, X + ((base_x ^ (kk << 5)) + mb * 32 * ROWB));
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  // The MFMAs of the k block in set s, with the operand reads of the NEXT k block (kk_next of slices Xr / Wr, into
+  // the other set) spread between them: one or two reads behind every pair of MFMAs.  The sched_barriers keep the
+  // compiler from gathering the reads (a burst of reads holds up the wave's MFMA issue) or sinking them to their use.
+  auto block = [&](int s, const unsigned char* Xr, const unsigned char* Wr, int kk_next, bool rd) __attribute__((always_inline)) {
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s][nb], xf[s][mb], acc[nb][mb], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (rd) {
+        wf[s ^ 1][nb] = *LDS_PTR(const bf16x8, Wr + ((base_w ^ (kk_next << 5)) + nb * 32 * ROWB));
+        if (nb < MB) xf[s ^ 1][nb] = *LDS_PTR(const bf16x8, Xr + ((base_x ^ (kk_next << 5)) + nb * 32 * ROWB));
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  // The loop is rotated so that the matrix pipe has work across the barrier: a step's last k block (operands already
+  // in registers) is multiplied AFTER the barrier that hands over the next slice, while the first operands of that
+  // slice are read.  Before the barrier a wave waits for its own LDS reads (the slot it read is overwritten by the
+  // loads issued after the barrier) and for its loads of the next slice.
   issue(0, sX0, sW0);
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(TOUCHES) : "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  fetch(sX0, sW0, 0, 0);
   auto step = [&](int ks, auto BUFC) __attribute__((always_inline)) {
     constexpr int BUF = decltype(BUFC)::value;
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (ks + 1 < n_steps) issue(ks + 1, BUF ? sX0 : sX1, BUF ? sW0 : sW1);
     const unsigned char* const X = BUF ? sX1 : sX0;
     const unsigned char* const W = BUF ? sW1 : sW0;
-    bf16x8 wf[2][4], xf[2][2];
-    auto fetch = [&](int kk, int s) __attribute__((always_inline)) {
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb) wf[s][nb] = *LDS_PTR(const bf16x8, W + ((base_w ^ (kk << 5)) + nb * 32 * ROWB));
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) xf[s][mb] = *LDS_PTR(const bf16x8, X + ((base_x ^ (kk << 5)) + mb * 32 * ROWB));
-    };
-    fetch(0, 0);
-#pragma unroll
-    for (int kk = 0; kk < 4; ++kk) {
-      if (kk + 1 < 4) fetch(kk + 1, (kk + 1) & 1);
-#pragma unroll
-      for (int nb = 0; nb < 4; ++nb)
-#pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
-          acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[kk & 1][nb], xf[kk & 1][mb], acc[nb][mb], 0, 0, 0);
-    }
+    unsigned char* const Xn = BUF ? sX0 : sX1;
+    unsigned char* const Wn = BUF ? sW0 : sW1;
+    const bool more = ks + 1 < n_steps;
+    if (more) issue(ks + 1, Xn, Wn);
+    __builtin_amdgcn_sched_barrier(0);
+    block(0, X, W, 1, true);
+    block(1, X, W, 2, true);
+    block(0, X, W, 3, true);
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(TOUCHES) : "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    block(1, Xn, Wn, 0, more);
   };
   int ks = 0;
   for (; ks + 1 < n_steps; ks += 2) {
@@ -151,8 +203,8 @@ __global__ __launch_bounds__(64 * NWAVES, 1) void qkv_gemm_prologue_kernel(const
   asm volatile("" : "+v"(lane_e));
   const int ie = lane_e & 31, ge = lane_e >> 5;
 #pragma unroll
-  for (int mb = 0; mb < 2; ++mb) {
-    const int s = m0 + 64 * wm + 32 * mb + ie;
+  for (int mb = 0; mb < MB; ++mb) {
+    const int s = m0 + 32 * MB * wm + 32 * mb + ie;
     const bool row_ok = s < a.S;
     // the projection's output is a bf16 tensor in the reference: round once, as it would have been
 #pragma unroll
@@ -253,12 +305,20 @@ hipError_t launch_qkv_gemm_prologue(const QkvGemmKernArgs& a_in, hipStream_t str
   QkvGemmKernArgs a = a_in;
   a.n_row_tiles = (a.S + BM - 1) / BM;
   a.n_col_tiles = (a.Hq + 2 * a.Hkv + a.Hqx) / 2;
-  const int lds = 4 * TILE;  // 128 KB of the CU's 160: above the default limit, asked for per launch (a host-side setting)
-  hipError_t e = hipFuncSetAttribute((const void*)qkv_gemm_prologue_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  const int lds = 4 * TILE + 1024;  // 129 KB of the CU's 160: above the default limit, asked for per launch (a host-side setting)
+#ifdef MAGI_TUNING
+  if (const char* v = getenv("MAGI_GEMM_WAVES")) a.variant = atoi(v);
+#endif
+  const bool four = a.variant == 4;  // (8 wavefronts of 128 x 64 unless a tuning build asks for 4 of 128 x 128)
+  const void* fn = four ? (const void*)qkv_gemm_prologue_kernel<4> : (const void*)qkv_gemm_prologue_kernel<2>;
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return e;
   const int supers = (a.n_row_tiles + 63) / 64;
   const unsigned grid = (unsigned)supers * 8u * 8u * (unsigned)a.n_col_tiles;
-  hipLaunchKernelGGL(qkv_gemm_prologue_kernel, dim3(grid), dim3(64 * NWAVES), lds, stream, a);
+  if (four)
+    hipLaunchKernelGGL(qkv_gemm_prologue_kernel<4>, dim3(grid), dim3(256), lds, stream, a);
+  else
+    hipLaunchKernelGGL(qkv_gemm_prologue_kernel<2>, dim3(grid), dim3(512), lds, stream, a);
   return hipGetLastError();
 }
 

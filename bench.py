@@ -352,6 +352,54 @@ def layer_norm_leg(inp, steps, traffic=None):
             "unit": "GB/s", "frac": round(gbs / PEAK_HBM_GBS, 4), "traffic": traffic, "ms": round(ms, 4)}
 
 
+def projection_leg(inp, steps):
+    """The four projections that feed the prologue (q, k, v and the cross-attention q: [S, hidden] x
+    [2 (Hq + Hkv) 128, hidden]^T), kernel-only and beside the headline: the library GEMM followed by the prologue
+    kernel (what the layer module runs) against the hand-written GEMM whose epilogue is the prologue
+    (magi_qkv_proj_prologue, the module's fused_projection option).  Same inputs, destinations of the step."""
+    import magi_attn as M
+
+    S, Hq, Hkv, D = inp["S"], inp["Hq"], inp["Hkv"], inp["D"]
+    hidden = Hq * D
+    dev = inp["q"].device
+    g = torch.Generator(device=dev).manual_seed(77)
+    x = inp["q_raw"]  # [S, hidden] bf16 N(0, 1): stands for the normalised hidden states
+    w = (torch.randn((2 * Hq + 2 * Hkv) * D, hidden, device=dev, generator=g) * hidden ** -0.5).bfloat16()
+    raw = torch.empty(S, w.shape[0], dtype=torch.bfloat16, device=dev)
+    z = inp["zeros"]
+    # destinations of their own (the step's q and cache rows still serve the CPU baseline's comparison)
+    q_dst = torch.empty_like(inp["q"])
+    kv_dst = torch.empty(S, Hkv, 2 * D, dtype=torch.bfloat16, device=dev)
+    nq, nk = Hq * D, Hkv * D
+    flop = 2.0 * S * hidden * w.shape[0]
+
+    def two_step():
+        torch.mm(x, w.t(), out=raw)
+        M.qk_prologue(raw[:, :nq], raw[:, nq:nq + nk], raw[:, nq + nk:nq + 2 * nk], inp["rope"], z, z, z, z, Hq=Hq, Hkv=Hkv,
+                      kv_out=kv_dst, n_cache_rows=S, q_out=q_dst, q_premul=Q_PREMUL)
+
+    def one_launch():
+        M.qkv_proj_prologue(x, w, inp["rope"], z, z, z, z, Hq=Hq, Hkv=Hkv, Hqx=Hq, kv_out=kv_dst, n_cache_rows=S,
+                            q_out=q_dst, qx_out=inp["xout"], q_premul=Q_PREMUL)
+
+    res = {"flop": flop, "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS}
+    for name, fn in (("library_gemm", lambda: torch.mm(x, w.t(), out=raw)), ("library_gemm_then_prologue", two_step),
+                     ("gemm_with_prologue_epilogue", one_launch)):
+        fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / steps
+        tf = flop / (ms * 1e-3) / 1e12
+        res[name] = {"ms": round(ms, 3), "achieved": round(tf, 1), "frac": round(tf / PEAK_BF16_TFLOPS, 4)}
+    res["what_the_layer_module_runs"] = "library_gemm_then_prologue"
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -365,6 +413,7 @@ def main():
                          "withholding the score bound, the online-softmax 32-row kernel that generic callers get")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-fp8", action="store_true")
+    ap.add_argument("--no-projection", action="store_true", help="skip the projection GEMM leg")
     ap.add_argument("--no-accuracy", action="store_true", help="skip the fp32 sampled-row check of the bf16 output")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="run one plain device copy of known size (for scaling FETCH_SIZE / WRITE_SIZE counters)")
@@ -459,6 +508,8 @@ def main():
         result["fp8"] = fp8_leg(inp, core_fl, core_tflops, args.steps, ref_rows, ref)
     result["roofline_layer_norm"] = layer_norm_leg(inp, args.steps, traffic.get("layer_norm"))
     result["roofline_layer_norm"]["traffic_source"] = TRAFFIC_SOURCE
+    if not args.no_projection:
+        result["projection"] = projection_leg(inp, args.steps)
     if args.copy_calibration:
         inp["q"].copy_(inp["out"])  # reads and writes out.numel() * 2 bytes each
         torch.cuda.synchronize()

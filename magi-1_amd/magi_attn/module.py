@@ -32,7 +32,8 @@ import math
 
 from . import _lib as L
 from .cache import Fp8KVCache
-from .functional import (head_norm, layer_norm, pow2_scale_for, qk_prologue, qk_prologue_fp8, quantize_fp8_split,
+from .functional import (head_norm, layer_norm, pow2_scale_for, qk_prologue, qk_prologue_fp8, qkv_proj_prologue,
+                         quantize_fp8_split,
                          range_attention)
 from .params import InferenceParams, ModelMetaArgs, PackedCrossAttnParams
 
@@ -170,12 +171,16 @@ class FullyParallelAttention(torch.nn.Module):
     def __init__(self, hidden_size: int, num_attention_heads: int, num_query_groups: int, kv_channels: int = 128,
                  layer_number: int = 0, layernorm_epsilon: float = 1e-6, apply_layernorm_1p: bool = True,
                  xattn_cond_hidden_ratio: float = 1.0, params_dtype=torch.bfloat16, device=None,
-                 attention_dtype: str = "bf16", fp8_fast_exp2: bool = True):
+                 attention_dtype: str = "bf16", fp8_fast_exp2: bool = True, fused_projection: bool = False):
         """attention_dtype "fp8" (not in the reference, which has no fp8 attention) runs the self-attention on
         e4m3 operands with per-(video chunk, head) power-of-two scales and keeps the KV cache in that form
         (Fp8KVCache); the cross attention and everything else stay in bf16.
         fp8_fast_exp2: the fp8 kernel's piecewise-linear exp2 (MAGI_ATTN_FP8_FAST_EXP2: about 10 % faster, the
-        output within the same accuracy bar as with the exact exponential); False for the exact one."""
+        output within the same accuracy bar as with the exact exponential); False for the exact one.
+        fused_projection: run the four projections and the prologue as ONE launch (magi_qkv_proj_prologue, the
+        hand-written GEMM whose epilogue is the prologue) instead of a library GEMM followed by the prologue kernel;
+        bf16 attention at batch 1 only.  Off by default: at the 720p shape the library GEMM + prologue take
+        10.9 ms, the fused launch 14.9 ms."""
         super().__init__()
         if kv_channels != 128:
             raise NotImplementedError("head_dim 128 only")
@@ -183,6 +188,7 @@ class FullyParallelAttention(torch.nn.Module):
             raise ValueError("attention_dtype must be 'bf16' or 'fp8'")
         self.attention_dtype = attention_dtype
         self.fp8_fast_exp2 = bool(fp8_fast_exp2)
+        self.fused_projection = bool(fused_projection)
         # forward() has the prologue fold softmax_scale * log2(e) into q ahead of q's one rounding to bf16 and tells
         # the attention kernel so (no per-score multiply there); get_q / get_qkv return q unscaled, as the reference
         self._q_premul = kv_channels ** -0.5 * math.log2(math.e)
@@ -547,9 +553,31 @@ class FullyParallelAttention(torch.nn.Module):
         sq = hidden_states.shape[0]
         D = self.hidden_size_per_attention_head
         mixed_qqkv = self.linear_qkv.forward_ln(hidden_states)
-        # all four projections in one GEMM; q / k / v feed the fused prologue as row-strided views of its result
-        q_raw, k_raw, v_raw, qx_raw = self.linear_qkv.forward_qkvx(mixed_qqkv)
-        raw = (q_raw, k_raw, v_raw)
+        one_launch = (self.fused_projection and self.attention_dtype == "bf16" and bs == 1 and rope is not None
+                      and rope.shape[-1] == 96 and mixed_qqkv.shape[-1] % 64 == 0)
+        if one_launch:
+            # projections + prologue in one launch: nothing raw reaches memory (qx leaves unnormalised, as the
+            # cross-attention kernel takes it)
+            raw = qx_raw = None
+        else:
+            # all four projections in one GEMM; q / k / v feed the fused prologue as row-strided views of its result
+            q_raw, k_raw, v_raw, qx_raw = self.linear_qkv.forward_qkvx(mixed_qqkv)
+            raw = (q_raw, k_raw, v_raw)
+
+        def project(kv_out=None, n_cache_rows=None, kv_tail=None):
+            """-> (q [S, Hq, D] carrying the softmax scale, kv destination(s), qx_raw [sq, 1, Hq*D])"""
+            if not one_launch:
+                q_, kv_ = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, kv_out=kv_out, n_cache_rows=n_cache_rows,
+                                          kv_tail=kv_tail, raw=raw, q_premul=self._q_premul, rope=rope)
+                return q_, kv_, qx_raw
+            gq_, bq_ = self.q_layernorm.gamma_beta_fp32()
+            gk_, bk_ = self.k_layernorm.gamma_beta_fp32()
+            q_, kv_, tail_, qx_ = qkv_proj_prologue(
+                mixed_qqkv.view(sq, -1), self.linear_qkv.fused_weight(), rope, gq_, bq_, gk_, bk_,
+                Hq=self.num_attention_heads, Hkv=self.num_query_groups_per_partition, Hqx=self.num_attention_heads,
+                eps=self.eps, kv_out=kv_out, n_cache_rows=n_cache_rows, kv_tail=kv_tail, q_premul=self._q_premul)
+            return q_, (kv_ if tail_ is None else (kv_, tail_)), qx_.view(sq, 1, -1)
+
         get_xqkv = lambda m, y: self.get_xqkv(m, y, qx_raw=qx_raw)
         p = meta_args.core_attn_params
         Hq = self.num_attention_heads
@@ -570,7 +598,7 @@ class FullyParallelAttention(torch.nn.Module):
             rope8 = rope if rope is not None else torch.cat([sin_emb, cos_emb], dim=-1).float().contiguous()
             core = self._core_attention_fp8(raw, rope8, inference_params, meta_args, use_cache, core_dst)
         elif not use_cache:
-            q, kv = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, raw=raw, q_premul=self._q_premul, rope=rope)
+            q, kv, qx_raw = project()
             core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst, q_prescaled=True,
                                        score_bound=bound_core)
         else:
@@ -593,8 +621,7 @@ class FullyParallelAttention(torch.nn.Module):
                     tail = torch.empty(S - n_keep, cache.shape[1], cache.shape[2], dtype=cache.dtype, device=cache.device)
                     self._kv_tail = tail
                 tail = tail[:S - n_keep]
-            q, _ = self._fused_qkv(mixed_qqkv, cos_emb, sin_emb, kv_out=cache[start:], n_cache_rows=n_keep,
-                                   kv_tail=tail, raw=raw, q_premul=self._q_premul, rope=rope)
+            q, _, qx_raw = project(kv_out=cache[start:], n_cache_rows=n_keep, kv_tail=tail)
             split = start + n_keep
             kc, vc = cache[:split, :, :D], cache[:split, :, D:]
             if tail is None:

@@ -45,69 +45,12 @@
 // laid out so that the workgroups an XCD receives (blockIdx % 8) share a KV head and walk the
 // same keys at about the same time (each XCD has its own L2).  Ranges are visited longest
 // first.  Fully masked key tiles never exist: a rectangle is walked from k_start to k_end only.
-#include "kernels.h"
-#include "wave_ops.h"
-
-#include <type_traits>
+#include "attn_common.h"
 
 namespace magi {
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef short s16x4 __attribute__((ext_vector_type(4)));
-typedef short s16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-
-#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
-#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
-
 constexpr int ROW_BYTES = 256;  // D = 128 bf16
-constexpr int MAX_SORT = 256;
-
-__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
-  f32x2 x = {a, b};
-  bf16x2 r = __builtin_convertvector(x, bf16x2);
-  return __builtin_bit_cast(unsigned, r);
-}
-
-__device__ __forceinline__ void load_range(const int* r, int mode, int i, int total, int& s, int& e) {
-  if (mode == 0) {
-    s = r[2 * i];
-    e = r[2 * i + 1];
-  } else {
-    s = r[i];
-    e = r[i + 1];
-  }
-  s = max(0, min(s, total));
-  e = max(s, min(e, total));
-}
-
-// f(integral_constant<int, I>) for I = B .. E-1, unrolled at compile time
-template <int B, int E, class F>
-__device__ __forceinline__ void static_for(F&& f) {
-  if constexpr (B < E) {
-    f(std::integral_constant<int, B>{});
-    static_for<B + 1, E>(f);
-  }
-}
-
-// s_waitcnt vmcnt(N), leaving the other counters alone
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
-  asm volatile("" ::: "memory");
-}
-
-// p0 + p1 + acc for a packed pair of bf16 values
-__device__ __forceinline__ float pair_sum(unsigned pk, float acc) {
-  const bf16x2 one = {(__bf16)1.0f, (__bf16)1.0f};
-  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), one, acc, false);
-}
 
 template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool PIPE = false, bool DB = false, bool PRESC = false>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
@@ -134,47 +77,11 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 
   const int tid = threadIdx.x;
   // ---- which piece of work is this workgroup? ----
-  const unsigned id = blockIdx.x;
-  const unsigned f = (id & 7u) * a.per_xcd + (id >> 3);
-  if (f >= a.total_wgs) return;
-  const unsigned per_range = (unsigned)a.tiles_per_range * (unsigned)a.G;
-  const unsigned per_kvh = (unsigned)a.n_ranges * per_range;
-  const unsigned kvh = f / per_kvh;
-  unsigned rem = f - kvh * per_kvh;
-  const unsigned rslot = rem / per_range;
-  rem -= rslot * per_range;
-  const unsigned tile = rem / (unsigned)a.G;
-  const unsigned hg = rem - tile * (unsigned)a.G;
-  const int h = (int)(kvh * a.G + hg);
-  // byte offset of this head in a row of `out` (optionally two-level: group, head in group)
-  const long o_head = a.out_group > 0 ? (long)(h / a.out_group) * a.os_g + (long)(h % a.out_group) * a.os_h : (long)h * a.os_h;
-
-  // range with the rslot-th longest key span (ties by index)
-  int ridx;
-  if (a.n_ranges <= MAX_SORT) {
-    if (tid < a.n_ranges) {
-      int s, e;
-      load_range(a.k_ranges, a.ranges_mode, tid, a.total_k, s, e);
-      const int my = e - s;
-      int rank = 0;
-      for (int j = 0; j < a.n_ranges; ++j) {
-        int sj, ej;
-        load_range(a.k_ranges, a.ranges_mode, j, a.total_k, sj, ej);
-        const int lj = ej - sj;
-        rank += (lj > my) || (lj == my && j < tid);
-      }
-      if (rank == (int)rslot) s_sel = tid;
-    }
-    __syncthreads();
-    ridx = __builtin_amdgcn_readfirstlane(s_sel);
-  } else {
-    ridx = a.n_ranges - 1 - (int)rslot;
-  }
-  int qs, qe, ks, ke;
-  load_range(a.q_ranges, a.ranges_mode, ridx, a.total_q, qs, qe);
-  load_range(a.k_ranges, a.ranges_mode, ridx, a.total_k, ks, ke);
-  const int q0 = qs + (int)tile * BM;
-  if (q0 >= qe) return;
+  const WorkItem wi = locate_work(a, BM, tid, &s_sel);
+  if (!wi.valid) return;
+  const int h = wi.h, q0 = wi.q0, qe = wi.qe, ks = wi.ks, ke = wi.ke;
+  const unsigned kvh = (unsigned)wi.kvh;
+  const long o_head = wi.o_head;
 
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l = tid & 63, i = l & 31, g = l >> 5;
@@ -182,12 +89,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   const bool row_ok = q_row < qe;
 
   if (ke <= ks) {  // no keys: zeros, lse = -inf
-    if (row_ok) {
-      char* op = a.out + (long)q_row * a.os_t + o_head + g * 128;
-#pragma unroll
-      for (int c = 0; c < 8; ++c) *(u32x4*)(op + c * 16) = u32x4{0, 0, 0, 0};
-      if (a.lse && g == 0) a.lse[(long)h * a.total_q + q_row] = -__builtin_inff();
-    }
+    if (row_ok) store_empty_row(a, wi, q_row, g);
     return;
   }
 

@@ -10,10 +10,7 @@
 //     segments), so inside a tile the K and V scales are wave-uniform scalars: the K scale joins
 //     the softmax scale, the V scale (relative to the largest V scale of the range) joins the exp2
 //     exponent, and the Q scale is a per-lane constant because a lane owns one query.
-#include "kernels.h"
-#include "wave_ops.h"
-
-#include <type_traits>
+#include "attn_common.h"
 
 namespace magi {
 namespace {
@@ -21,41 +18,14 @@ namespace {
 typedef int i32x8 __attribute__((ext_vector_type(8)));
 typedef int i32x2 __attribute__((ext_vector_type(2)));
 typedef int i32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
-typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
-
-#define LDS_PTR(T, p) ((T __attribute__((address_space(3)))*)(p))
-#define GLOBAL_PTR(p) ((const __attribute__((address_space(1))) void*)(p))
 
 constexpr int BN = 64;
 constexpr int ROW_BYTES = 128;  // D = 128 fp8
 constexpr int TILE_BYTES = BN * ROW_BYTES;
-constexpr int MAX_SORT = 256;
 constexpr int NW = 4;
 constexpr int BM = 32 * NW;
 constexpr int LOADS = 8 / NW;  // direct loads per wave per matrix per tile (8 rows each)
 constexpr float P_SHIFT = 8.f;
-
-__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {
-  f32x2 x = {a, b};
-  bf16x2 r = __builtin_convertvector(x, bf16x2);
-  return __builtin_bit_cast(unsigned, r);
-}
-
-__device__ __forceinline__ void load_range(const int* r, int mode, int i, int total, int& s, int& e) {
-  if (mode == 0) {
-    s = r[2 * i];
-    e = r[2 * i + 1];
-  } else {
-    s = r[i];
-    e = r[i + 1];
-  }
-  s = max(0, min(s, total));
-  e = max(s, min(e, total));
-}
 
 // FASTP (with POW2): the probabilities come from a piecewise-linear exp2 built on the matrix pipe's scaling
 // instead of the quarter-rate v_exp_f32 (see the softmax below).
@@ -72,46 +42,10 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
-  const unsigned id = blockIdx.x;
-  const unsigned f = (id & 7u) * a.per_xcd + (id >> 3);
-  if (f >= a.total_wgs) return;
-  const unsigned per_range = (unsigned)a.tiles_per_range * (unsigned)a.G;
-  const unsigned per_kvh = (unsigned)a.n_ranges * per_range;
-  const unsigned kvh = f / per_kvh;
-  unsigned rem = f - kvh * per_kvh;
-  const unsigned rslot = rem / per_range;
-  rem -= rslot * per_range;
-  const unsigned tile = rem / (unsigned)a.G;
-  const unsigned hg = rem - tile * (unsigned)a.G;
-  const int h = (int)(kvh * a.G + hg);
-  // byte offset of this head in a row of `out` (optionally two-level: group, head in group)
-  const long o_head = a.out_group > 0 ? (long)(h / a.out_group) * a.os_g + (long)(h % a.out_group) * a.os_h : (long)h * a.os_h;
-
-  int ridx;
-  if (a.n_ranges <= MAX_SORT) {
-    if (tid < a.n_ranges) {
-      int s, e;
-      load_range(a.k_ranges, a.ranges_mode, tid, a.total_k, s, e);
-      const int my = e - s;
-      int rank = 0;
-      for (int j = 0; j < a.n_ranges; ++j) {
-        int sj, ej;
-        load_range(a.k_ranges, a.ranges_mode, j, a.total_k, sj, ej);
-        const int lj = ej - sj;
-        rank += (lj > my) || (lj == my && j < tid);
-      }
-      if (rank == (int)rslot) s_sel = tid;
-    }
-    __syncthreads();
-    ridx = __builtin_amdgcn_readfirstlane(s_sel);
-  } else {
-    ridx = a.n_ranges - 1 - (int)rslot;
-  }
-  int qs, qe, ks, ke;
-  load_range(a.q_ranges, a.ranges_mode, ridx, a.total_q, qs, qe);
-  load_range(a.k_ranges, a.ranges_mode, ridx, a.total_k, ks, ke);
-  const int q0 = qs + (int)tile * BM;
-  if (q0 >= qe) return;
+  const WorkItem wi = locate_work(a, BM, tid, &s_sel);
+  if (!wi.valid) return;
+  const int h = wi.h, kvh = wi.kvh, q0 = wi.q0, qe = wi.qe, ks = wi.ks, ke = wi.ke;
+  const long o_head = wi.o_head;
 
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int l = tid & 63, i = l & 31, g = l >> 5;
@@ -119,12 +53,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   const bool row_ok = q_row < qe;
 
   if (ke <= ks) {
-    if (row_ok) {
-      char* op = a.out + (long)q_row * a.os_t + o_head + g * 128;
-#pragma unroll
-      for (int c = 0; c < 8; ++c) *(u32x4*)(op + c * 16) = u32x4{0, 0, 0, 0};
-      if (a.lse && g == 0) a.lse[(long)h * a.total_q + q_row] = -__builtin_inff();
-    }
+    if (row_ok) store_empty_row(a, wi, q_row, g);
     return;
   }
 

@@ -218,6 +218,8 @@ def apply_rotary_emb(x, cos, sin, interleaved=False, inplace=False, **_unused):
     R2 = cos.shape[-1]
     if cos.shape != (S, R2) or sin.shape != (S, R2):
         raise ValueError("cos / sin must be [seqlen, rotary_dim / 2]")
+    if inplace and not x.is_contiguous():
+        raise ValueError("inplace=True needs a contiguous x (a copy would be rotated instead of x)")
     xc = x.contiguous()
     y = xc if inplace else torch.empty_like(xc)
     cosf = cos.to(torch.float32).contiguous()

@@ -173,6 +173,12 @@ def test_apply_rotary_emb_matches_oracle(dev):
     yb = M.apply_rotary_emb(x.bfloat16().to(dev), cos.to(dev), sin.to(dev))
     assert (yb.float().cpu() - O.apply_rope_neox_partial(x.bfloat16().float(), cos, sin)).abs().max() < 2e-2
     assert torch.equal(yb[..., 96:].cpu(), x.bfloat16()[..., 96:])
+    # in place: the tensor itself is rotated; a strided view cannot be (a copy would be rotated instead)
+    xi = x.to(dev).clone()
+    assert M.apply_rotary_emb(xi, cos.to(dev), sin.to(dev), inplace=True).data_ptr() == xi.data_ptr()
+    assert torch.equal(xi, y)
+    with pytest.raises(ValueError):
+        M.apply_rotary_emb(x.to(dev).transpose(1, 2).contiguous().transpose(1, 2), cos.to(dev), sin.to(dev), inplace=True)
 
 
 def test_rejects_bad_arguments(dev):

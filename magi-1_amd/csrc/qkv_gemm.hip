@@ -37,7 +37,7 @@ constexpr int R2 = 48;  // rotary pairs (the MAGI-1 layout: rotary_dim 96 of 128
 
 // MB: blocks of 32 tokens per wavefront.  MB = 2 (shipped): 8 wavefronts (two per SIMD), 128 accumulator registers
 // each.  MB = 4: 4 wavefronts (one per SIMD) with 256 accumulator registers each, 0.5 instead of 0.75 KB of LDS
-// operand reads per MFMA, but nothing to hide a wave's own waits behind; measured 2 % slower.
+// operand reads per MFMA, but nothing to hide a wave's own waits behind; measured within 2 % of the other.
 template <int MB>
 __global__ __launch_bounds__(64 * (16 / MB), 1) void qkv_gemm_prologue_kernel(const QkvGemmKernArgs a) {
   constexpr int NWAVES = 16 / MB;
@@ -80,20 +80,19 @@ __global__ __launch_bounds__(64 * (16 / MB), 1) void qkv_gemm_prologue_kernel(co
   const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc((void*)wb, 0, 0x7fffffff, 0x00020000);
   const unsigned vx = (unsigned)(8 * w + lr) * (unsigned)a.x_stride + (unsigned)(chunk * 16);
   const unsigned vw = (unsigned)(8 * w + lr) * (unsigned)a.w_stride + (unsigned)(chunk * 16);
-  auto issue = [&](int kstep, unsigned char* sX, unsigned char* sW) __attribute__((always_inline)) {
+  auto issue_pair = [&](int j, int kstep, unsigned char* sX, unsigned char* sW) __attribute__((always_inline)) {
     const unsigned kb = (unsigned)kstep * (unsigned)ROWB;
-#pragma unroll
-    for (int j = 0; j < LOADS; ++j) {
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, LDS_PTR(void, sX + (w + NWAVES * j) * 1024), 16, vx,
-                                               (int)(kb + (unsigned)(8 * NWAVES * j) * (unsigned)a.x_stride), 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, LDS_PTR(void, sW + (w + NWAVES * j) * 1024), 16, vw,
-                                               (int)(kb + (unsigned)(8 * NWAVES * j) * (unsigned)a.w_stride), 0, 0);
-    }
-    // Warm the caches for the slice after that one: one 4-byte load per 128-byte row segment, issued BEHIND the
-    // loads above (loads complete in order, so the wait in front of the barrier can leave exactly these
-    // outstanding) into LDS that nothing reads.  A slice is requested by the ~32 workgroups of an XCD at about the
-    // same time and the first request goes to HBM (measured: 6 % on the 4-wavefront form, which has nothing to
-    // hide a wait behind; no difference on the 8-wavefront form).
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, LDS_PTR(void, sX + (w + NWAVES * j) * 1024), 16, vx,
+                                             (int)(kb + (unsigned)(8 * NWAVES * j) * (unsigned)a.x_stride), 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, LDS_PTR(void, sW + (w + NWAVES * j) * 1024), 16, vw,
+                                             (int)(kb + (unsigned)(8 * NWAVES * j) * (unsigned)a.w_stride), 0, 0);
+  };
+  // Warm the caches for the slice after `kstep`: one 4-byte load per 128-byte row segment, issued BEHIND the loads of
+  // slice `kstep` (loads complete in order, so the wait in front of the barrier can leave exactly these outstanding)
+  // into LDS that nothing reads.  A slice is requested by the ~32 workgroups of an XCD at about the same time and
+  // the first request goes to HBM (measured: 6 % on the 4-wavefront form, which has nothing to hide a wait behind;
+  // no difference on the 8-wavefront form).  Always issued: the waits count them.
+  auto issue_touch = [&](int kstep) __attribute__((always_inline)) {
     const unsigned kt = (unsigned)min(kstep + 1, n_steps - 1) * (unsigned)ROWB;
     if constexpr (MB == 4) {
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, LDS_PTR(void, sJunk), 4, (unsigned)tid * (unsigned)a.x_stride, (int)kt, 0, 0);
@@ -128,20 +127,34 @@ __global__ __launch_bounds__(64 * (16 / MB), 1) void qkv_gemm_prologue_kernel(co
     for (int mb = 0; mb < MB; ++mb) xf[s][mb] = *LDS_PTR(const bf16x8, X + ((base_x ^ (kk << 5)) + mb * 32 * ROWB));
     __builtin_amdgcn_sched_barrier(0);
   };
-  // The MFMAs of the k block in set s, with the operand reads of the NEXT k block (kk_next of slices Xr / Wr, into
-  // the other set) spread between them: one or two reads behind every pair of MFMAs.  The sched_barriers keep the
-  // compiler from gathering the reads (a burst of reads holds up the wave's MFMA issue) or sinking them to their use.
-  auto block = [&](int s, const unsigned char* Xr, const unsigned char* Wr, int kk_next, bool rd) __attribute__((always_inline)) {
+  // The MFMAs of the k block in set s in four groups (one feature block each), and behind every group a share of the
+  // other work, so that the wave never goes long without issuing an MFMA:
+  //  * the operand reads of the NEXT k block (kk_next of slices Xr / Wr, into the other set): the token fragments
+  //    first, because the next block's first group needs all of them, then the feature fragments in the order of use;
+  //  * if ld0 >= 0, the direct loads of the next slice: wave-load pairs ld0 + group, and behind the last pair the
+  //    cache-warming loads.
+  // The sched_barriers keep the compiler from gathering all this or sinking a read to its use.
+  auto block = [&](int s, const unsigned char* Xr, const unsigned char* Wr, int kk_next, bool rd, int ld0 = -100,
+                   int kstep = 0, unsigned char* Xl = nullptr, unsigned char* Wl = nullptr) __attribute__((always_inline)) {
+    constexpr int NREAD = MB + 4;  // fragments per k block: x0 .. x(MB-1), w0 .. w3
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) {
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
+      for (int mb = 0; mb < MB; ++mb) {
         acc[nb][mb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf[s][nb], xf[s][mb], acc[nb][mb], 0, 0, 0);
+      }
       __builtin_amdgcn_sched_barrier(0);
       if (rd) {
-        wf[s ^ 1][nb] = *LDS_PTR(const bf16x8, Wr + ((base_w ^ (kk_next << 5)) + nb * 32 * ROWB));
-        if (nb < MB) xf[s ^ 1][nb] = *LDS_PTR(const bf16x8, Xr + ((base_x ^ (kk_next << 5)) + nb * 32 * ROWB));
+#pragma unroll
+        for (int r = nb * NREAD / 4; r < (nb + 1) * NREAD / 4; ++r) {
+          if (r < MB)
+            xf[s ^ 1][r] = *LDS_PTR(const bf16x8, Xr + ((base_x ^ (kk_next << 5)) + r * 32 * ROWB));
+          else
+            wf[s ^ 1][r - MB] = *LDS_PTR(const bf16x8, Wr + ((base_w ^ (kk_next << 5)) + (r - MB) * 32 * ROWB));
+        }
       }
+      if (ld0 + nb >= 0 && ld0 + nb < LOADS && kstep < n_steps) issue_pair(ld0 + nb, kstep, Xl, Wl);
+      if (ld0 + nb == LOADS - 1) issue_touch(kstep);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -149,7 +162,9 @@ __global__ __launch_bounds__(64 * (16 / MB), 1) void qkv_gemm_prologue_kernel(co
   // in registers) is multiplied AFTER the barrier that hands over the next slice, while the first operands of that
   // slice are read.  Before the barrier a wave waits for its own LDS reads (the slot it read is overwritten by the
   // loads issued after the barrier) and for its loads of the next slice.
-  issue(0, sX0, sW0);
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j) issue_pair(j, 0, sX0, sW0);
+  issue_touch(0);
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(TOUCHES) : "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
@@ -161,10 +176,8 @@ __global__ __launch_bounds__(64 * (16 / MB), 1) void qkv_gemm_prologue_kernel(co
     unsigned char* const Xn = BUF ? sX0 : sX1;
     unsigned char* const Wn = BUF ? sW0 : sW1;
     const bool more = ks + 1 < n_steps;
-    if (more) issue(ks + 1, Xn, Wn);
-    __builtin_amdgcn_sched_barrier(0);
-    block(0, X, W, 1, true);
-    block(1, X, W, 2, true);
+    block(0, X, W, 1, true, 0, ks + 1, Xn, Wn);
+    block(1, X, W, 2, true, LOADS > 4 ? 4 : -100, ks + 1, Xn, Wn);
     block(0, X, W, 3, true);
     asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(TOUCHES) : "memory");
     __builtin_amdgcn_s_barrier();

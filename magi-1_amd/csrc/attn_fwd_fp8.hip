@@ -28,7 +28,7 @@ constexpr int LOADS = 8 / NW;  // direct loads per wave per matrix per tile (8 r
 constexpr float P_SHIFT = 8.f;
 
 // FASTP (with POW2): the probabilities come from a piecewise-linear exp2 built on the matrix pipe's scaling
-// instead of the quarter-rate v_exp_f32 (see the softmax below).
+// instead of the quarter-rate v_exp_f32: the score registers hold e4m3 codes (see the softmax below).
 template <bool POW2, bool FASTP = false>
 __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKernArgs a) {
   // Two (K tile, V tile) buffers as four separate objects that are only ever indexed statically: the compiler
@@ -162,13 +162,15 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   // row's maximum; there m starts at 0 and the first tile sets it.
   float m_run = POW2 ? 0.f : -__builtin_inff();
   float l_run = 0.f;
-  // FASTP: the score MFMAs carry 23 more on their scale exponent and accumulate onto (127 + shift - m) * 2^23, so a
-  // register holds (e + 127) * 2^23 for the exponent e of its probability: truncated to an integer that is the bit
-  // pattern of the fp32 number 2^floor(e) * (1 + frac(e)), exp2 with a linear mantissa (at most 6.2 % above 2^e,
-  // 4 % on average; the row sum is taken from the same values, so the average cancels and a relative spread of
-  // 2 % is what remains, beside the 2.7 % of the rounding to e4m3).  One full-rate conversion per score.
-  constexpr float XS = FASTP ? 8388608.f : 1.f;       // units of the accumulator per exponent unit
-  constexpr float XB = FASTP ? 127.f * 8388608.f : 0.f;  // accumulator value of exponent 0
+  // FASTP: the score MFMAs carry 3 more on their scale exponent and accumulate onto (7 + shift - m) * 8, so a
+  // register holds 8 (e + 7) for the exponent e of its probability.  An e4m3 code c above 7 stands for
+  // 2^(c / 8 - 7) * (1 + (c % 8) / 8), so that register, converted to an integer, IS the e4m3 code of exp2 with a linear
+  // mantissa (at most 6.2 % above 2^e) on a grid of an eighth of an octave: one full-rate convert-and-insert per
+  // score (v_cvt_pk_u8_f32; it saturates at 0, and the row maximum keeps the codes at or below 120 = 2^8).  The row
+  // sum is taken from the same codes on the matrix pipe, so the average excess cancels in the normalisation.
+  constexpr float XS = FASTP ? 8.f : 1.f;   // units of the accumulator per exponent unit
+  constexpr float XB = FASTP ? 56.f : 0.f;  // accumulator value of exponent 0
+  constexpr int XE = FASTP ? 3 : 0;         // log2(XS), carried by the key scale's exponent
   f32x16 neg_m;
 #pragma unroll
   for (int v = 0; v < 16; ++v) neg_m[v] = XB;
@@ -176,6 +178,14 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   bool first = true;
   const int e_q = (__builtin_bit_cast(int, q_sc) >> 23) & 0xff;  // E8M0 code of the (power-of-two) query scale
   const bool wave_on = (q0 + 32 * w) < qe;
+  // Selector rows of the row-sum MFMA (16x16x128, half the time of a 32x32x64 one).  Read as the B operand of that
+  // shape, the P registers of lane l are column l % 16, and of the 128 products of a column they are numbers
+  // 16 (l / 16) .. + 15 (registers 0-3) and 64 + 16 (l / 16) .. + 15 (registers 4-7): queries j and j + 16 share column j
+  // in alternating runs of 16.  An fp4 A operand holds products 32 (l / 16) .. + 31 of row l % 16 in four registers, the
+  // first two covering a run of query j, the last two one of query j + 16.  Rows 0 and 8 of A are 1.0 (fp4 e2m1
+  // 0b0010) on the runs of j, rows 4 and 12 on those of j + 16, all else 0, and register 0 of the result of lane l is
+  // row 4 (l / 16) of column l % 16: the sum over all 64 keys of the query the lane holds.
+  const int ones_lo = (l & 7) == 0 ? 0x22222222 : 0, ones_hi = (l & 7) == 4 ? 0x22222222 : 0;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const float c_q = a.scale_log2 * q_sc;  // softmax scale * log2(e) * q scale
 
@@ -214,7 +224,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         if constexpr (!POW2) c = c_q * k_sc;                             // per-lane score scale inside this piece
         shift = uni(P_SHIFT + __builtin_amdgcn_logf(v_sc) - log2_vmax);  // <= 8
         unshift = uni(__builtin_amdgcn_exp2f(-shift));
-        e_k = ((__builtin_bit_cast(int, k_sc) >> 23) & 0xff) + (FASTP ? 23 : 0);  // E8M0 code of a power-of-two key scale
+        e_k = ((__builtin_bit_cast(int, k_sc) >> 23) & 0xff) + XE;  // E8M0 code of a power-of-two key scale
       }
 
       auto read_k = [&](int t, int kk) -> i32x8 {
@@ -248,7 +258,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         }
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-          s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[0], qf[0], neg_m, 0, 0, 0, e_k, 0, e_q);  // (FASTP: e_k carries + 23)
+          s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[0], qf[0], neg_m, 0, 0, 0, e_k, 0, e_q);  // (FASTP: e_k carries + 3)
           if (t == 0) ka[0] = read_k(1, 0);
           __builtin_amdgcn_sched_barrier(0);  // (keeps each operand read one MFMA ahead of its use, where it is written)
           s_acc[t] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ka[1], qf[1], s_acc[t], 0, 0, 0, e_k, 0, e_q);
@@ -277,7 +287,6 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
             if (key >= pe) s_acc[t][v] = -__builtin_inff();
           }
       }
-      float psum = 0.f, psum2 = 0.f;
       float mx = max3(s_acc[0][0], s_acc[0][1], s_acc[0][2]);
 #pragma unroll
       for (int t = 0; t < 2; ++t)
@@ -307,30 +316,25 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           }
         }
         first = false;
-        auto pexp = [](float x) -> float {
-          if constexpr (FASTP) {  // (the conversion saturates at 0 for negative values and -inf: a probability of 0)
-            float r;
-            asm("v_cvt_u32_f32 %0, %1" : "=v"(r) : "v"(x));
-            return r;
-          } else
-            return __builtin_amdgcn_exp2f(x);
-        };
 #pragma unroll
         for (int n = 0; n < 8; ++n) {  // dword n = slots 4n .. 4n+3 = s_acc[n >> 2][4 (n & 3) .. +3]
-          const float p0 = pexp(s_acc[n >> 2][4 * (n & 3) + 0]);
-          const float p1 = pexp(s_acc[n >> 2][4 * (n & 3) + 1]);
-          const float p2 = pexp(s_acc[n >> 2][4 * (n & 3) + 2]);
-          const float p3 = pexp(s_acc[n >> 2][4 * (n & 3) + 3]);
-          if constexpr (FASTP) {  // row sum by vector additions (see the row-sum MFMA below)
-            psum += p0 + p1;
-            psum2 += p2 + p3;
+          const float x0 = s_acc[n >> 2][4 * (n & 3) + 0], x1 = s_acc[n >> 2][4 * (n & 3) + 1];
+          const float x2 = s_acc[n >> 2][4 * (n & 3) + 2], x3 = s_acc[n >> 2][4 * (n & 3) + 3];
+          if constexpr (FASTP) {  // (the conversion saturates at 0 for negative values and -inf: a probability of 0)
+            unsigned u = __builtin_amdgcn_cvt_pk_u8_f32(x0, 0, 0u);
+            u = __builtin_amdgcn_cvt_pk_u8_f32(x1, 1, u);
+            u = __builtin_amdgcn_cvt_pk_u8_f32(x2, 2, u);
+            pb[n] = (int)__builtin_amdgcn_cvt_pk_u8_f32(x3, 3, u);
+          } else {
+            const float p0 = __builtin_amdgcn_exp2f(x0), p1 = __builtin_amdgcn_exp2f(x1);
+            const float p2 = __builtin_amdgcn_exp2f(x2), p3 = __builtin_amdgcn_exp2f(x3);
+            // v_cvt_pk_fp8_f32 keeps the other half of its destination: start from p0's register (its high half is
+            // overwritten by the second conversion) instead of a zeroed one
+            int u = __builtin_bit_cast(int, p0);
+            u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
+            u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
+            pb[n] = u;
           }
-          // v_cvt_pk_fp8_f32 keeps the other half of its destination: start from p0's register (its high half is
-          // overwritten by the second conversion) instead of a zeroed one
-          int u = __builtin_bit_cast(int, p0);
-          u = __builtin_amdgcn_cvt_pk_fp8_f32(p0, p1, u, false);
-          u = __builtin_amdgcn_cvt_pk_fp8_f32(p2, p3, u, true);
-          pb[n] = u;
         }
       } else {
         const float m_new = fmaxf(m_run, mx * c);
@@ -360,21 +364,16 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         va[0] = read_v(0);
         va[1] = read_v(1);
       }
-      // Row sums on the matrix pipe: ones^T P^T.  One more MFMA per tile (A = 1.0 in every position, written as fp4
-      // so that it takes four registers; it and the result live in the score registers, which are dead by now)
-      // instead of 32 vector additions per lane: this kernel is bound by vector-instruction issue (its 32
-      // exponentials alone take as long as its 8 MFMAs), not by the matrix pipe.  Every row of the product is the
-      // sum over all 64 keys of the probabilities AS ROUNDED to e4m3, i.e. of exactly what the PV product uses, and
-      // both lanes of a query get the full sum.  Issued ahead of the PV MFMAs and read after them.
-      // With FASTP the vector pipe has room again (one full-rate conversion per score instead of a quarter-rate
-      // exponential), so the row sum goes back to it (32 additions per lane of the values ahead of their rounding
-      // to e4m3, whose rounding errors average out over a row) and the matrix pipe keeps to its 8 MFMAs.
+      // Row sums on the matrix pipe: one more, half-length MFMA per tile (selector rows times P^T, see `ones_lo`; A in
+      // fp4 so that it takes four registers) instead of 32 vector additions per lane.  The sum is over the
+      // probabilities AS ROUNDED to e4m3, i.e. of exactly what the PV product uses, and both lanes of a query get the
+      // full sum.  Issued ahead of the PV MFMAs and read after them.
       __builtin_amdgcn_sched_barrier(0);
       i32x8 ones;
 #pragma unroll
-      for (int n = 0; n < 8; ++n) ones[n] = n < 4 ? 0x22222222 : 0;  // fp4 e2m1 1.0 = 0b0010
-      f32x16 rowsum = zero16;
-      if constexpr (!FASTP) rowsum = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(ones, pb, zero16, 4, 0, 0, 0, 0, 0);
+      for (int n = 0; n < 8; ++n) ones[n] = n < 2 ? ones_lo : n < 4 ? ones_hi : 0;
+      f32x4 rowsum = {0.f, 0.f, 0.f, 0.f};
+      rowsum = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pb, rowsum, 4, 0, 0, 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) {  // two V operands in flight, in alternating registers
@@ -382,7 +381,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         if (mb + 2 < 4) va[mb & 1] = read_v(mb + 2);
       }
       __builtin_amdgcn_sched_barrier(0);
-      l_run += (FASTP ? psum + psum2 : rowsum[0]) * unshift;
+      l_run += rowsum[0] * unshift;
     }
     k0 = k1;
     pe = pe1;
@@ -397,9 +396,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   }
 
   if (!wave_on) return;
-  // (the row-sum MFMA hands every lane the sum over all keys of its query; the vector sums of FASTP cover the keys
-  // of the lane's own half wave)
-  const float l_tot = FASTP ? l_run + __shfl_xor(l_run, 32) : l_run;
+  const float l_tot = l_run;  // (the row-sum MFMA hands every lane the sum over all keys of its query)
   const float inv = v_max * __builtin_amdgcn_exp2f(-P_SHIFT) / l_tot;
   // A lane holds four consecutive features per (mb, b), its partner in the other half wave the next four: the
   // halves trade the odd-b registers of the lower half for the even-b registers of the upper one, after which

@@ -238,7 +238,8 @@ def test_attention_kernels_keep_their_registers():
     """A register spill inside a tile loop costs a drain of the tile loads per tile (parity stays green while the
     launch runs 1.7x slower), and the allocator decides per instantiation: compile the attention sources for
     gfx950 and check the compiler's own resource report.  The bf16 instantiations must use no scratch memory at
-    all; the fp8 kernel is allowed its known 16 bytes (three values parked across the loop, not inside it)."""
+    all; the fp8 kernel is allowed its known 24 bytes (values parked across the loop and reloaded on the ragged-tile
+    path and in the epilogue, not in the steady-state loop)."""
     import shutil
     import subprocess
 
@@ -251,7 +252,7 @@ def test_attention_kernels_keep_their_registers():
              "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage", "-c", "-o", os.devnull]
     # the 64-row kernel: no scratch at all in the plain instantiations; the one that normalises q while loading it
     # (template arguments <..., false, true>, mangled ...ELb0ELb1EE) may park values around that prologue, outside the loop
-    for src, limit in (("attn_fwd_bf16.hip", 0), ("attn_fwd_fp8.hip", 16), ("attn_fwd_bf16_w64.hip", 0)):
+    for src, limit in (("attn_fwd_bf16.hip", 0), ("attn_fwd_fp8.hip", 24), ("attn_fwd_bf16_w64.hip", 0)):
         r = subprocess.run([hipcc] + flags + [os.path.join(csrc, src)], capture_output=True, text=True, timeout=600)
         assert r.returncode == 0, r.stderr[-2000:]
         names = re.findall(r"Function Name: (\S+)", r.stderr)

@@ -221,6 +221,51 @@ def test_fp8_scores_far_below_zero_from_the_first_tile(dev, pow2):
     assert err <= 4e-2 and cos >= 0.998, (err, cos)
 
 
+@pytest.mark.parametrize("pow2", [False, True, "fast_exp2"])
+def test_fp8_row_maximum_rising_late_and_often(dev, pow2):
+    """Keys whose scores climb along the key axis: a key aligned with the queries every 70 keys, each ~25 octaves above
+    the one before, so that the running maximum is raised in tile after tile (ragged last tile included) and what
+    was accumulated before each raise has to be scaled away.  The last aligned key ends up with all the weight."""
+    fast = pow2 == "fast_exp2"
+    pow2 = bool(pow2)
+    g = torch.Generator().manual_seed(78)
+    T, Tk, Hq, Hkv, D = 96, 333, 2, 1, 128
+    sign = torch.where(torch.rand(D, generator=g) < 0.5, -1.0, 1.0)
+    q = (1.0 * sign + 0.05 * torch.randn(T, Hq, D, generator=g)).bfloat16()
+    k = (0.05 * torch.randn(Tk, Hkv, D, generator=g))
+    steps = list(range(20, Tk, 70))
+    for n, j in enumerate(steps):
+        k[j] += (n + 1) * 1.5 * sign  # score (n + 1) * 1.5 * 128 / sqrt(128) * log2(e) = 24.5 (n + 1) in base-2 units
+    k = k.bfloat16()
+    v = torch.randn(Tk, Hkv, D, generator=g).bfloat16()
+    qr, kr = [[0, T]], [[0, Tk]]
+    cs = D ** -0.5 * math.log2(math.e)
+    C = 128  # three scale chunks along the keys, the last one partial
+    q8, qs = M.quantize_fp8(q.to(dev), C, premul=cs if pow2 else 1.0, pow2_scales=pow2)
+    k8, ks = M.quantize_fp8(k.to(dev), C, pow2_scales=pow2)
+    v8, vs = M.quantize_fp8(v.to(dev), C, pow2_scales=pow2)
+    tq = torch.tensor(qr, dtype=torch.int32, device=dev)
+    tk = torch.tensor(kr, dtype=torch.int32, device=dev)
+    out, lse = M.range_attention(q8, k8, v8, tq, tk, T, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=C,
+                                 fp8_pow2_prescaled=pow2, fp8_fast_exp2=fast)
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    qd = O.dequantize_per_head_chunk(q8.cpu(), qs.cpu(), C)
+    kd = O.dequantize_per_head_chunk(k8.cpu(), ks.cpu(), C)
+    vd = O.dequantize_per_head_chunk(v8.cpu(), vs.cpu(), C)
+    if pow2:
+        ref = O.range_attention(qd / cs * D ** -0.5, kd, vd, qr, kr, softmax_scale=1.0)
+        ref_lse = O.range_attention_lse(qd / cs * D ** -0.5, kd, vd, qr, kr, softmax_scale=1.0)
+    else:
+        ref = O.range_attention(qd, kd, vd, qr, kr)
+        ref_lse = O.range_attention_lse(qd, kd, vd, qr, kr)
+    err, cos = _per_head(out, ref)
+    assert err <= 4e-2 and cos >= 0.9995, (err, cos)
+    # one key holds the weight: the output is its V row and lse its score (base e), ~ 24.5 * 5 * ln 2 = 85
+    last = steps[-1]
+    assert (out.float().cpu() - vd[last, 0].float()).abs().max() <= 4e-2
+    assert (lse.cpu() - ref_lse).abs().max() <= (8.5e-2 if fast else 2e-2) and ref_lse.min() > 60
+
+
 def test_fp8_uneven_scales_and_two_segments(dev):
     """Chunks with very different magnitudes (the per-chunk scales must be honoured, including the
     relative V scale folded into the exponent) and a key axis split over two buffers."""

@@ -168,6 +168,8 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   // mantissa (at most 6.2 % above 2^e) on a grid of an eighth of an octave: one full-rate convert-and-insert per
   // score (v_cvt_pk_u8_f32; it saturates at 0, and the row maximum keeps the codes at or below 120 = 2^8).  The row
   // sum is taken from the same codes on the matrix pipe, so the average excess cancels in the normalisation.
+  // (Measured and dropped: v_cvt_pknorm_u16_f32 on pairs of scores and one v_perm_b32 per four for their high bytes,
+  // 3 instructions per 4 scores instead of 4, is 20 % slower: those two do not issue at the full rate.)
   constexpr float XS = FASTP ? 8.f : 1.f;   // units of the accumulator per exponent unit
   constexpr float XB = FASTP ? 56.f : 0.f;  // accumulator value of exponent 0
   constexpr int XE = FASTP ? 3 : 0;         // log2(XS), carried by the key scale's exponent
@@ -175,9 +177,9 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
 #pragma unroll
   for (int v = 0; v < 16; ++v) neg_m[v] = XB;
   float cur_shift = 0.f;
-  bool first = true;
+  int first = 1;  // (wave-uniform, kept as an integer so that it lives in a scalar register) no tile seen yet
   const int e_q = (__builtin_bit_cast(int, q_sc) >> 23) & 0xff;  // E8M0 code of the (power-of-two) query scale
-  const bool wave_on = (q0 + 32 * w) < qe;
+  const bool wave_on = __builtin_amdgcn_readfirstlane(q0 + 32 * w) < __builtin_amdgcn_readfirstlane(qe);  // (a scalar condition)
   // Selector rows of the row-sum MFMA (16x16x128, half the time of a 32x32x64 one).  Read as the B operand of that
   // shape, the P registers of lane l are column l % 16, and of the 128 products of a column they are numbers
   // 16 (l / 16) .. + 15 (registers 0-3) and 64 + 16 (l / 16) .. + 15 (registers 4-7): queries j and j + 16 share column j
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         if constexpr (!POW2) c = c_q * k_sc;                             // per-lane score scale inside this piece
         shift = uni(P_SHIFT + __builtin_amdgcn_logf(v_sc) - log2_vmax);  // <= 8
         unshift = uni(__builtin_amdgcn_exp2f(-shift));
-        e_k = ((__builtin_bit_cast(int, k_sc) >> 23) & 0xff) + XE;  // E8M0 code of a power-of-two key scale
+        e_k = max(((__builtin_bit_cast(int, k_sc) >> 23) & 0xff) + XE, 0);  // E8M0 code of a power-of-two key scale
       }
 
       auto read_k = [&](int t, int kk) -> i32x8 {
@@ -296,10 +298,12 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       if constexpr (POW2) {
         // s_acc already holds exponent - m_run + shift; a value above `shift` is a new row maximum
         const float over = mx - (shift * XS + XB);
-        const bool raise = first || over > 0.f;
-        if (__builtin_amdgcn_ballot_w64(raise) != 0) {
-          const float delta = raise ? over : 0.f;
-          const float alpha = first ? 1.f : __builtin_amdgcn_exp2f(-delta * (1.f / XS));  // nothing to rescale on the first tile
+        const bool up = over > 0.f;
+        int any_up;  // (scalar test of the lane mask; the compiler's own goes through two vector instructions)
+        asm("s_cmp_lg_u64 %1, 0\n\ts_cselect_b32 %0, 1, 0" : "=s"(any_up) : "s"(__builtin_amdgcn_ballot_w64(up)) : "scc");
+        if ((first | any_up) != 0) {
+          const float delta = (first != 0 || up) ? over : 0.f;
+          const float alpha = first != 0 ? 1.f : __builtin_amdgcn_exp2f(-delta * (1.f / XS));  // nothing to rescale on the first tile
           m_run += delta * (1.f / XS);
           l_run *= alpha;
 #pragma unroll
@@ -308,14 +312,14 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           for (int t = 0; t < 2; ++t)
 #pragma unroll
             for (int v = 0; v < 16; ++v) s_acc[t][v] -= delta;
-          if (!first) {
+          if (first == 0) {
 #pragma unroll
             for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
               for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
           }
         }
-        first = false;
+        first = 0;
 #pragma unroll
         for (int n = 0; n < 8; ++n) {  // dword n = slots 4n .. 4n+3 = s_acc[n >> 2][4 (n & 3) .. +3]
           const float x0 = s_acc[n >> 2][4 * (n & 3) + 0], x1 = s_acc[n >> 2][4 * (n & 3) + 1];
@@ -374,6 +378,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       for (int n = 0; n < 8; ++n) ones[n] = n < 2 ? ones_lo : n < 4 ? ones_hi : 0;
       f32x4 rowsum = {0.f, 0.f, 0.f, 0.f};
       rowsum = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(ones, pb, rowsum, 4, 0, 0, 0, 0, 0);
+      asm volatile("" : "+v"(rowsum));  // (an empty statement that holds the MFMA here: left alone it sinks to its use, and the wave waits there)
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int mb = 0; mb < 4; ++mb) {  // two V operands in flight, in alternating registers

@@ -11,8 +11,9 @@ namespace magi {
 // wait states that the compiler inserts for the builtin.
 __device__ __forceinline__ float half_swap_max(float x) {
   float lo = x, hi = x;
-  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(lo), "+v"(hi));
-  return fmaxf(lo, hi);
+  // (the maximum inside the statement: fmaxf would first quiet both operands, two more instructions)
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1\n\tv_max_f32 %0, %0, %1" : "+v"(lo), "+v"(hi));
+  return lo;
 }
 
 // Exchange lanes 32..63 of `a` with lanes 0..31 of `b` (both must be VALU results, see above).

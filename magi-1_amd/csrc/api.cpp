@@ -195,6 +195,12 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     a.variant = env_variant;
 #endif
   }
+#ifdef MAGI_TUNING
+  if (p->dtype == MAGI_DTYPE_FP8_E4M3) {
+    static const int env_variant8 = tuning_env("MAGI_ATTN_VARIANT");
+    a.variant = env_variant8;
+  }
+#endif
   a.tiles_per_range = (p->max_seqlen_q + a.block_m - 1) / a.block_m;
   a.Hq = p->Hq;
   a.Hkv = p->Hkv;

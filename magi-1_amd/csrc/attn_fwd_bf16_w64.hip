@@ -51,7 +51,9 @@ __device__ __forceinline__ float keep_lanes(float p, unsigned long long m) {
   return r;
 }
 
-template <int NW, int OCC, bool BOUNDED, int VPRE, int RD, bool PIPE = false, bool QNORM = false>
+// WHATIF (tuning builds only, timing only: the results are wrong): parts of the bounded softmax left out, to measure
+// what each costs.  1: no exponentials, 2: no row-sum additions.
+template <int NW, int OCC, bool BOUNDED, int VPRE, int RD, bool PIPE = false, bool QNORM = false, int WHATIF = 0>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const AttnKernArgs a) {
   constexpr int BM = 64 * NW;
   constexpr int LW = 4;                 // waves that load tiles (the last LW of the workgroup)
@@ -253,7 +255,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const A
           // halves keep their value is a scalar question per register
           const int left = ke - kbase;  // valid keys in this half (may be <= 0)
           auto prob = [&](float x, int v) __attribute__((always_inline)) -> float {
-            const float p = __builtin_amdgcn_exp2f(x);
+            const float p = (WHATIF & 1) ? x : __builtin_amdgcn_exp2f(x);
             if constexpr (RAGGED) {
               const int c0 = 8 * (v >> 2) + (v & 3);
               const unsigned long long m = (c0 < left ? 0x00000000ffffffffull : 0ull) | (c0 + 4 < left ? 0xffffffff00000000ull : 0ull);
@@ -272,11 +274,13 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const A
 #pragma unroll
               for (int e = 0; e < 16; e += 2) {
                 const float p0 = prob(sc[b][e], e), p1 = prob(sc[b][e + 1], e + 1);
-                psum += p0;
-                psum2 += p1;
+                if constexpr (!(WHATIF & 2)) {
+                  psum += p0;
+                  psum2 += p1;
+                }
                 sc[b][8 * (e >> 3) + ((e & 7) >> 1)] = __builtin_bit_cast(float, pack_bf16x2(p0, p1));
               }
-              l_run[b] += psum + psum2;
+              l_run[b] += ((WHATIF & 2) ? 1.f : 0.f) + psum + psum2;
             } else {
               float mx = max3(sc[b][0], sc[b][1], sc[b][2]);
 #pragma unroll
@@ -615,7 +619,11 @@ hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream) {
   hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<NW, OCC, true, VPRE, RD>), dim3(grid), dim3(64 * NW), 0, stream, a)
 #endif
 #ifdef MAGI_TUNING
-  if (a.variant == 20)  // software-pipelined loop, one wave per SIMD
+  if (a.variant >= 101 && a.variant <= 103 && bounded) {  // MAGI_ATTN_VARIANT = 100 + WHATIF
+    if (a.variant == 101) hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 2, true, 0, 4, false, false, 1>), dim3(grid), dim3(256), 0, stream, a);
+    if (a.variant == 102) hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 2, true, 0, 4, false, false, 2>), dim3(grid), dim3(256), 0, stream, a);
+    if (a.variant == 103) hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 2, true, 0, 4, false, false, 3>), dim3(grid), dim3(256), 0, stream, a);
+  } else if (a.variant == 20)  // software-pipelined loop, one wave per SIMD
     hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 1, true, 0, 4, true>), dim3(grid), dim3(256), 0, stream, a);
   else if (a.block_m == 512 && a.variant == 12)
     MAGI_W64_LAUNCH(8, 1, 0, 2);

@@ -251,7 +251,7 @@ def test_attention_kernels_keep_their_registers():
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
              "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage", "-c", "-o", os.devnull]
     # the 64-row kernel: no scratch at all in the plain instantiations; the one that normalises q while loading it
-    # (template arguments <..., false, true>, mangled ...ELb0ELb1EE) may park values around that prologue, outside the loop
+    # (template arguments <..., false, true, 0>, mangled ...ELb0ELb1ELi0EE) may park values around that prologue, outside the loop
     for src, limit in (("attn_fwd_bf16.hip", 0), ("attn_fwd_fp8.hip", 24), ("attn_fwd_bf16_w64.hip", 0)):
         r = subprocess.run([hipcc] + flags + [os.path.join(csrc, src)], capture_output=True, text=True, timeout=600)
         assert r.returncode == 0, r.stderr[-2000:]
@@ -263,7 +263,7 @@ def test_attention_kernels_keep_their_registers():
         for n, sc, vg in zip(names, scratch, vgprs):
             if "attn_fwd" in n:
                 seen += 1
-                lim = 128 if (src == "attn_fwd_bf16_w64.hip" and n.endswith("ELb0ELb1EEEvNS_12AttnKernArgsE")) else limit
+                lim = 128 if (src == "attn_fwd_bf16_w64.hip" and n.endswith("ELb0ELb1ELi0EEEvNS_12AttnKernArgsE")) else limit
                 assert sc <= lim, f"{n}: {sc} bytes of scratch per lane"
                 assert vg <= 256
         assert seen >= 2

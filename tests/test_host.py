@@ -29,6 +29,25 @@ def test_library_loads_and_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_missing_library_is_an_error_not_a_fallback(tmp_path):
+    """The library named by MAGI_ATTN_LIBRARY is the one that is loaded; when it does not exist the first call
+    raises (there is no other compute path to fall back to)."""
+    import subprocess
+    import sys
+
+    code = (
+        "import sys; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+        "import magi_attn._lib as L\n"
+        "try:\n"
+        "    L.lib()\n"
+        "except RuntimeError as e:\n"
+        "    assert 'no fallback' in str(e), e; print('raised')\n"
+    ) % (os.path.join(ROOT, "magi-1_amd"), ROOT)
+    env = dict(os.environ, MAGI_ATTN_LIBRARY=str(tmp_path / "absent" / "libmagi_attn.so"))
+    r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
+    assert r.returncode == 0 and r.stdout.strip() == "raised", (r.stdout, r.stderr[-2000:])
+
+
 def test_struct_layouts_match_header(tmp_path):
     """ctypes mirrors vs the C compiler's view of include/magi_attn.h (sizes and field offsets)."""
     import subprocess

@@ -403,7 +403,7 @@ def projection_leg(inp, steps):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=2)
     ap.add_argument("--workload", default="720p-24B", choices=sorted(WORKLOADS))
     ap.add_argument("--kv-window", default="default", choices=["default", "noise2clean"],

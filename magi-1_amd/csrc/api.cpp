@@ -40,15 +40,6 @@ int compute_units() {
   return cached[dev];
 }
 
-#ifdef MAGI_TUNING
-// Tuning builds only (make TUNING=1): MAGI_ATTN_BLOCK_M / MAGI_ATTN_VARIANT pick a bf16 kernel instantiation by hand
-// for A/B measurements.  Read once per process; the shipped library has no such knobs.
-int tuning_env(const char* name) {
-  const char* e = std::getenv(name);
-  return e ? std::atoi(e) : 0;
-}
-#endif
-
 }  // namespace
 
 extern "C" {
@@ -109,8 +100,8 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     if (!aligned16(p->q_norm_gamma) || !aligned16(p->q_norm_beta))
       return fail(MAGI_EINVAL, "magi_attn_fwd: q_norm parameters must be 16-byte aligned");
   }
-  if (p->score_bound > 0.f && !q_norm && !(p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)))
-    return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound needs bf16 inputs with MAGI_ATTN_Q_PRESCALED (or q_norm)");
+  if (p->score_bound > 0.f && p->dtype != MAGI_DTYPE_BF16)
+    return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound is a promise about bf16 inputs");
   if (p->out_group_heads < 0 || (p->out_group_heads > 0 && (p->Hq % p->out_group_heads || p->o_stride_g % 8)))
     return fail(MAGI_EINVAL, "magi_attn_fwd: out_group_heads must divide Hq and o_stride_g keep rows 16-byte aligned");
   int k_split = p->total_k;
@@ -175,6 +166,9 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   if (p->dtype == MAGI_DTYPE_FP8_E4M3 && p->q_tile_rows != 0 && p->q_tile_rows != 128)
     return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (fp8: 128)", p->q_tile_rows);
   const bool bounded = p->dtype == MAGI_DTYPE_BF16 && p->score_bound > 0.f && p->score_bound <= MAGI_SCORE_BOUND_MAX;
+  // a bound stated for unscaled q (what the reference's callers pass): the kernel applies the softmax scale while it
+  // loads q, after which the scores are exp2 exponents as with MAGI_ATTN_Q_PRESCALED
+  const bool scale_q = bounded && !q_norm && !(p->flags & MAGI_ATTN_Q_PRESCALED);
   if (p->dtype == MAGI_DTYPE_BF16) {
     const double wg384 = (double)p->Hq * p->n_ranges * ((p->max_seqlen_q + 383) / 384);
     const bool long_keys = p->max_seqlen_k == 0 || p->max_seqlen_k >= 4096;  // (0 = not stated)
@@ -184,23 +178,13 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
       a.block_m = 384;
     if (p->q_tile_rows != 0) {
       const int r = p->q_tile_rows;
-      if (q_norm && r != 256) return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (with q_norm: 256)", r);
+      if ((q_norm || scale_q) && r != 256)
+        return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (with q_norm, or a score bound on unscaled q: 256)", r);
       if (bounded ? (r != 256 && r != 512) : (r != 128 && r != 384))
         return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (bf16: 128 or 384; with a score bound: 256 or 512)", r);
       a.block_m = r;
     }
-#ifdef MAGI_TUNING
-    static const int env_block_m = tuning_env("MAGI_ATTN_BLOCK_M"), env_variant = tuning_env("MAGI_ATTN_VARIANT");
-    if (env_block_m == 128 || env_block_m == 256 || env_block_m == 384 || env_block_m == 512) a.block_m = env_block_m;
-    a.variant = env_variant;
-#endif
   }
-#ifdef MAGI_TUNING
-  if (p->dtype == MAGI_DTYPE_FP8_E4M3) {
-    static const int env_variant8 = tuning_env("MAGI_ATTN_VARIANT");
-    a.variant = env_variant8;
-  }
-#endif
   a.tiles_per_range = (p->max_seqlen_q + a.block_m - 1) / a.block_m;
   a.Hq = p->Hq;
   a.Hkv = p->Hkv;
@@ -212,7 +196,7 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     a.k2_scale_delta = (p->k2_scale - p->k_scale) - (long)a.scale_split_chunk * p->Hkv;
     a.v2_scale_delta = (p->v2_scale - p->v_scale) - (long)a.scale_split_chunk * p->Hkv;
   }
-  a.flags = p->flags | (bounded ? magi::ATTN_BOUNDED : 0);
+  a.flags = p->flags | (bounded ? magi::ATTN_BOUNDED : 0) | (scale_q ? magi::ATTN_SCALE_Q : 0);
   const double total = (double)p->Hq * p->n_ranges * a.tiles_per_range;
   if (total > 2.0e9) return fail(MAGI_EINVAL, "magi_attn_fwd: grid too large (%.3g workgroups)", total);
   a.total_wgs = (unsigned)total;
@@ -220,12 +204,13 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 1.0f / std::sqrt((float)p->D);
   a.scale_log2 = scale * 1.4426950408889634f;
   if (p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)) a.scale_log2 = 1.f;  // q . k is the exp2 exponent
-  // (with q_norm the kernel multiplies the normalised q by scale_log2 itself, after which the same holds)
+  // (with q_norm, or a score bound on unscaled q, the kernel multiplies q by scale_log2 itself while loading it, after
+  // which the same holds)
 
   hipError_t e;
   if (p->dtype != MAGI_DTYPE_BF16)
     e = magi::launch_attn_fwd_fp8(a, static_cast<hipStream_t>(stream));
-  else if (bounded || a.variant >= 10)
+  else if (bounded)
     e = magi::launch_attn_fwd_bf16_w64(a, static_cast<hipStream_t>(stream));
   else
     e = magi::launch_attn_fwd_bf16(a, static_cast<hipStream_t>(stream));

@@ -36,10 +36,6 @@
 // Operand reads from LDS are written a few MFMAs ahead of their use and held there with scheduling
 // barriers (the instruction scheduler otherwise sinks them to one MFMA ahead); the epilogue trades
 // registers between the half waves so that every lane stores 16 contiguous bytes.
-// Instantiations with 2 waves / SIMD (deep prefetch, K and V double buffered), with 32-key tiles,
-// with 8-wave workgroups, and a software-pipelined loop (PIPE: score MFMAs of the next tile, softmax
-// and PV MFMAs of the current one interleaved in one basic block, 2 waves / SIMD) are kept for
-// comparison; on the 720p layer none is faster.
 //
 // Work decomposition: blockIdx -> (kv head, range slot, q tile, q head within the GQA group),
 // laid out so that the workgroups an XCD receives (blockIdx % 8) share a KV head and walk the
@@ -52,7 +48,8 @@ namespace {
 
 constexpr int ROW_BYTES = 256;  // D = 128 bf16
 
-template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool PIPE = false, bool DB = false, bool PRESC = false>
+// VSINGLE: the 4-wave form (two K slots, one V slot); DB: the 12-wave form (K and V double buffered); exactly one of them
+template <int NW, int BN, int NSTAGE, int OCC, bool VSINGLE, bool DB = false, bool PRESC = false>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnKernArgs a) {
   constexpr int BM = 32 * NW;
   constexpr int TILE_BYTES = BN * ROW_BYTES;
@@ -68,11 +65,8 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   constexpr bool VMID = DB && PRESC;           // ... in the middle of the softmax (V is in LDS by then only in the DB loop)
   static_assert(LOADS >= 1 && NSTAGE >= 2 && NSTAGE <= 4, "bad tile configuration");
   static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");
-  static_assert(!PIPE || (NSTAGE == 2 && BN == 64 && !VSINGLE), "pipelined loop: 64-key tiles, two K slots and two V slots");
-  static_assert(!DB || (NSTAGE == 2 && !VSINGLE && !PIPE), "static double buffer: two K slots and two V slots");
-  // ring of NSTAGE (K tile, V tile) pairs for the loops that index their slots at run time; the single-V, the
-  // double-buffered and the pipelined loops declare their slots as separate objects and leave this one a stub
-  __shared__ __attribute__((aligned(1024))) unsigned char smem[(PIPE || DB || VSINGLE) ? 1 : 2 * NSTAGE][(PIPE || DB || VSINGLE) ? 16 : TILE_BYTES];
+  static_assert(!DB || (NSTAGE == 2 && !VSINGLE), "static double buffer: two K slots and two V slots");
+  static_assert(DB != VSINGLE, "one of the two tile loops");
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -166,10 +160,6 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       }
     }
   };
-  auto issue_tile = [&](int k0, int stage) {
-    issue_mat(k0, &smem[2 * stage][0], false);
-    issue_mat(k0, &smem[2 * stage + 1][0], true);
-  };
 
   // ---- per-lane LDS read bases ----
   // K as A operand: row = 32t + i, 16-byte chunk 2kk + g  ->  off = base_k ^ (kk << 5), + t * 32 rows
@@ -198,184 +188,6 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
   const int n_tiles = (ke - ks + BN - 1) / BN;
-  if constexpr (PIPE) {
-    // Software-pipelined loop.  Iteration `it` runs, in ONE basic block, the score MFMAs of tile it+1, the
-    // exp2 / pack / row-sum work of tile it, the PV MFMAs of tile it and the row max of tile it+1, cut into
-    // 32 chunks of one MFMA + its operand reads + a few VALU instructions each (scheduling barriers pin the
-    // chunks), so that the VALU work issues in the shadow of the MFMAs of the same wave.  The lazy rescale of
-    // O and the tail mask sit between iterations.  K(t) lives in K slot t & 1, V(t) in V slot t & 1; the loads
-    // for K(it+2) and V(it+1) are issued at the top of iteration it and have the whole iteration to land.
-    // The four slots are four separate LDS objects and the loop is unrolled by two so that every access names
-    // its slot statically: the compiler then knows that the operand reads of an iteration never touch the
-    // slots the in-flight direct loads write, and does not make the reads wait for those loads.
-    __shared__ __attribute__((aligned(1024))) unsigned char sK0[TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) unsigned char sK1[TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) unsigned char sV0[TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) unsigned char sV1[TILE_BYTES];
-    auto read_k = [&](const unsigned char* Kt, int idx) -> bf16x8 {  // idx = 8t + kk
-      return *LDS_PTR(const bf16x8, Kt + ((base_k ^ ((idx & 7) << 5)) + (idx >> 3) * 32 * ROW_BYTES));
-    };
-    auto read_v = [&](const unsigned char* Vt, int p) -> bf16x8 {  // p = 4 * slab + mb
-      const int mb = p & 3, sl = p >> 2;
-      const int bv = base_v ^ (mb << 6);
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * sl) * ROW_BYTES)));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (16 * sl + 8) * ROW_BYTES)));
-      const s16x8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-      return __builtin_bit_cast(bf16x8, va);
-    };
-    constexpr int PD = 4;  // operand reads in flight (2 .. 8 measure the same)
-    f32x16 sA[2], sB[2];   // scores of even / odd tiles
-    float m_new, alpha;
-
-    // ---- prologue: K(0) -> scores of tile 0 and their row max ----
-    issue_mat(ks, sK0, false);
-    wait_vmcnt<0>();
-    __syncthreads();
-    if (n_tiles > 1) issue_mat(ks + BN, sK1, false);
-    issue_mat(ks, sV0, true);
-    {
-      bf16x8 kbuf[PD];
-#pragma unroll
-      for (int idx = 0; idx < PD; ++idx) kbuf[idx] = read_k(sK0, idx);
-#pragma unroll
-      for (int idx = 0; idx < 16; ++idx) {
-        const int t = idx >> 3, kk = idx & 7;
-        sA[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kbuf[idx % PD], qf[kk], kk == 0 ? zero16 : sA[t], 0, 0, 0);
-        if (idx + PD < 16) kbuf[idx % PD] = read_k(sK0, idx + PD);
-      }
-      // keys past the end of the range repeat the last valid row (the loader clamps), so the max needs no mask
-      float mx = sA[0][0];
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) mx = fmaxf(mx, sA[t][v]);
-      m_new = half_swap_max(mx);
-      alpha = 0.f;
-    }
-
-    // between iterations (tile `it` of parity P): lazy rescale, tail mask, publish the next tiles
-    auto top = [&](int it, auto pc, f32x16 (&s_cur)[2]) {
-      constexpr int P = decltype(pc)::value;
-      const int k0 = ks + it * BN;
-      if (it > 0 && __builtin_amdgcn_ballot_w64(alpha != 1.f) != 0) {  // some row of this wave saw a new maximum
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) o_acc[mb][v] *= alpha;
-      }
-      if (k0 + BN > ke) {  // ragged last tile: keys >= ke do not exist
-#pragma unroll
-        for (int t = 0; t < 2; ++t)
-#pragma unroll
-          for (int v = 0; v < 16; ++v) {
-            const int key = k0 + 32 * t + 8 * (v >> 2) + 4 * g + (v & 3);
-            if (key >= ke) s_cur[t][v] = -__builtin_inff();
-          }
-      }
-      wait_vmcnt<0>();
-      __syncthreads();  // K(it+1) and V(it) landed; K slot P and V slot P^1 are free
-      if (it + 2 < n_tiles) issue_mat(k0 + 2 * BN, P ? sK1 : sK0, false);
-      if (it + 1 < n_tiles) issue_mat(k0 + BN, P ? sV0 : sV1, true);
-    };
-    constexpr int SM_OPS = 96;
-
-    // one pipelined iteration for a tile of parity P
-    auto step = [&](int it, auto pc, f32x16 (&s_cur)[2], f32x16 (&s_nxt)[2]) {
-      constexpr int P = decltype(pc)::value;
-      top(it, pc, s_cur);
-      if (!wave_on) return;
-      const unsigned char* Kn = P ? sK0 : sK1;
-      const unsigned char* Vt = P ? sV1 : sV0;
-      const float mc = m_new * c;
-      const float m_prev = m_new;  // running max including tile it
-
-      float psum = 0.f;
-      float mxa = 0.f, mxb = 0.f, m_nx = 0.f, al_nx = 1.f;
-      // softmax micro-ops of tile it: group j = elements (2j, 2j+1) of the 32 this lane holds, 6 ops per group
-      // (the packed probabilities of slab s overwrite the first four of the eight score registers they came
-      // from, so P needs no registers of its own)
-      auto sm_op = [&](auto nc) {
-        constexpr int n = decltype(nc)::value;
-        constexpr int j = n / 6, k = n % 6;
-        constexpr int t = j >> 3, v0 = 2 * (j & 7);
-        constexpr int pw = 8 * ((j >> 2) & 1) + (j & 3);  // register of s_cur[t] that receives packed pair j
-        if constexpr (k == 0) s_cur[t][v0] = fmaf(s_cur[t][v0], c, -mc);
-        if constexpr (k == 1) s_cur[t][v0 + 1] = fmaf(s_cur[t][v0 + 1], c, -mc);
-        if constexpr (k == 2) s_cur[t][v0] = __builtin_amdgcn_exp2f(s_cur[t][v0]);
-        if constexpr (k == 3) s_cur[t][v0 + 1] = __builtin_amdgcn_exp2f(s_cur[t][v0 + 1]);
-        if constexpr (k == 4) s_cur[t][pw] = __builtin_bit_cast(float, pack_bf16x2(s_cur[t][v0], s_cur[t][v0 + 1]));
-        if constexpr (k == 5) {
-          const float packed = s_cur[t][pw];  // (a bit_cast applied to the vector element itself reads element 0)
-          psum = pair_sum(__builtin_bit_cast(unsigned, packed), psum);
-        }
-      };
-      auto p_operand = [&](int sl) -> bf16x8 {  // B operand of the PV MFMAs for slab sl
-        const f32x16& sv = s_cur[sl >> 1];
-        const f32x4 r = (sl & 1) ? __builtin_shufflevector(sv, sv, 8, 9, 10, 11) : __builtin_shufflevector(sv, sv, 0, 1, 2, 3);
-        return __builtin_bit_cast(bf16x8, r);
-      };
-      // row-max micro-ops of tile it+1: 8 + 8 max3, then combine / running max / alpha
-      auto mr_op = [&](auto nc) {
-        constexpr int n = decltype(nc)::value;
-        constexpr int q = n & 7;
-        if constexpr (n < 16) {
-          const f32x16& sv = s_nxt[n >> 3];
-          float& m = (n < 8) ? mxa : mxb;
-          if constexpr (q == 0) m = max3(sv[0], sv[1], sv[2]);
-          else if constexpr (q < 7) m = max3(m, sv[2 * q + 1], sv[2 * q + 2]);
-          else m = max3(m, sv[15], sv[15]);
-        } else if constexpr (n == 16) {
-          m_nx = half_swap_max(max3(mxa, mxb, mxb));
-        } else if constexpr (n == 17) {
-          m_nx = max3(m_prev, m_nx, m_nx);
-        } else if constexpr (n == 18) {
-          al_nx = __builtin_amdgcn_exp2f((m_prev - m_nx) * c);
-        }
-      };
-      bf16x8 obuf[PD];  // operand ring: K operands during the score MFMAs, then V operands
-#pragma unroll
-      for (int idx = 0; idx < PD; ++idx) obuf[idx] = read_k(Kn, idx);
-      // VALU work that does not wait for the operand reads
-      static_for<0, 6>(sm_op);
-      __builtin_amdgcn_sched_barrier(0);
-      static_for<0, 32>([&](auto chc) {
-        constexpr int ch = decltype(chc)::value;
-        if constexpr (ch < 16) {
-          constexpr int t = ch >> 3, kk = ch & 7;
-          s_nxt[t] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(obuf[ch % PD], qf[kk], kk == 0 ? zero16 : s_nxt[t], 0, 0, 0);
-          if constexpr (ch + PD < 16)
-            obuf[ch % PD] = read_k(Kn, ch + PD);
-          else
-            obuf[ch % PD] = read_v(Vt, ch + PD - 16);
-        } else {
-          constexpr int p = ch - 16;
-          o_acc[p & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(obuf[ch % PD], p_operand(p >> 2), o_acc[p & 3], 0, 0, 0);
-          if constexpr (p + PD < 16) obuf[ch % PD] = read_v(Vt, p + PD);
-        }
-        // softmax ops: all 96 done after chunk 25 (slab 3 is needed by chunk 28)
-        constexpr int lo = 6 + (90 * ch) / 26, hi0 = 6 + (90 * (ch + 1)) / 26, hi = hi0 < SM_OPS ? hi0 : SM_OPS;
-        static_for<(lo < hi ? lo : hi), hi>(sm_op);
-        // row max of tile it+1: first half of the scores is complete after chunk 7, the second after chunk 15
-        if constexpr (ch >= 10 && ch < 18) mr_op(std::integral_constant<int, ch - 10>{});
-        if constexpr (ch >= 19 && ch < 27) mr_op(std::integral_constant<int, ch - 19 + 8>{});
-        if constexpr (ch >= 28 && ch < 31) mr_op(std::integral_constant<int, ch - 28 + 16>{});
-        __builtin_amdgcn_sched_barrier(0);
-      });
-      l_run = l_run * alpha + psum;
-      m_run = m_prev;
-      m_new = m_nx;
-      alpha = al_nx;
-    };
-    // The last tile runs the same step: its score MFMAs read a K slot that holds no new tile and produce
-    // values nobody uses (one wasted product per workgroup instead of a second copy of the loop body).
-    const std::integral_constant<int, 0> even;
-    const std::integral_constant<int, 1> odd;
-    for (int it = 0; it < n_tiles; it += 2) {
-      step(it, even, sA, sB);
-      if (it + 1 >= n_tiles) break;
-      step(it + 1, odd, sB, sA);
-    }
-  } else {
   // One key tile for this wave: scores, online softmax, PV.  Kt / Vt: the tile's K and V slots; before_pv runs
   // between the softmax and the first V operand read (the single-V mode publishes V(it) there).
   auto compute_tile = [&](const unsigned char* Kt, const unsigned char* Vt, int k0, auto before_pv) {
@@ -583,36 +395,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
       if (it + 1 >= n_tiles) break;
       step(it + 1, std::integral_constant<int, 1>{});
     }
-  } else {
-    // ring of NSTAGE (K tile, V tile) pairs, tiles requested NSTAGE-1 ahead, one barrier per tile
-#pragma unroll
-    for (int p = 0; p < NSTAGE - 1; ++p)
-      if (p < n_tiles) issue_tile(ks + p * BN, p);
-    int stage = 0;
-    for (int it = 0; it < n_tiles; ++it) {
-      const int k0 = ks + it * BN;
-      // tile `it` must have landed; up to NSTAGE-2 younger tiles may still be in flight
-      const int younger = min(NSTAGE - 2, n_tiles - 1 - it);
-      if (NSTAGE >= 4 && younger == 2)
-        wait_vmcnt<2 * TILE_LOADS>();
-      else if (NSTAGE >= 3 && younger == 1)
-        wait_vmcnt<TILE_LOADS>();
-      else
-        wait_vmcnt<0>();
-      __syncthreads();  // everybody's share landed; the stage read in the previous iteration is free again
-      if (it + NSTAGE - 1 < n_tiles) {
-        int st = stage + NSTAGE - 1;
-        if (st >= NSTAGE) st -= NSTAGE;
-        issue_tile(k0 + (NSTAGE - 1) * BN, st);
-      }
-      const unsigned char* Kt = &smem[2 * stage][0];
-      const unsigned char* Vt = &smem[2 * stage + 1][0];
-      stage = (stage + 1 == NSTAGE) ? 0 : stage + 1;
-      if (!wave_on) continue;
-      compute_tile(Kt, Vt, k0, []() {});
-    }
-  }  // !DB
-  }  // !PIPE
+  }
 
   if (!wave_on) return;
   // ---- epilogue: normalise and store ----
@@ -649,34 +432,16 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
 }  // namespace
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream) {
-  const unsigned grid = a.per_xcd * 8u;
+  const dim3 grid(a.per_xcd * 8u);
   const bool presc = (a.flags & 2) != 0;  // q pre-scaled: the scores are exp2 exponents (PRESC instantiations)
-#ifdef MAGI_TUNING
-  // comparison instantiations, reachable in tuning builds only (MAGI_ATTN_BLOCK_M / MAGI_ATTN_VARIANT)
-  if (a.block_m == 256 && a.variant == 3)  // software-pipelined loop, 8 waves, 256 query rows, 2 waves / SIMD
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false, true>), dim3(grid), dim3(512), 0, stream, a);
-  else if (a.block_m == 256)  // 8 waves, 256 query rows, 2 waves / SIMD
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<8, 64, 2, 2, false>), dim3(grid), dim3(512), 0, stream, a);
-  else if (a.block_m == 128 && a.variant == 1)  // 32-key tiles, 3-stage ring, 3 waves / SIMD
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 32, 3, 3, false>), dim3(grid), dim3(256), 0, stream, a);
-  else if (a.block_m == 128 && a.variant == 2)  // 64-key tiles, double-buffered K and V, 2 waves / SIMD
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false>), dim3(grid), dim3(256), 0, stream, a);
-  else if (a.block_m == 128 && a.variant == 3)  // software-pipelined loop, 2 waves / SIMD
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 2, false, true>), dim3(grid), dim3(256), 0, stream, a);
-  else if (a.block_m == 384 && a.variant == 7)  // pre-scaled q through the instantiation with the per-score multiply
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true>), dim3(grid), dim3(768), 0, stream, a);
-  else if (a.variant == 7)
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), dim3(grid), dim3(256), 0, stream, a);
-  else
-#endif
   if (a.block_m == 384 && presc)  // 12 waves, 384 query rows, one workgroup per CU = 3 waves / SIMD sharing every tile
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true, true>), dim3(grid), dim3(768), 0, stream, a);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, true, true>), grid, dim3(768), 0, stream, a);
   else if (a.block_m == 384)
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, false, true>), dim3(grid), dim3(768), 0, stream, a);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<12, 64, 2, 1, false, true>), grid, dim3(768), 0, stream, a);
   else if (presc)  // 4 waves, 64-key tiles, double-buffered K, single V slot, three workgroups per CU
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true, false, false, true>), dim3(grid), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true, false, true>), grid, dim3(256), 0, stream, a);
   else
-    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), dim3(grid), dim3(256), 0, stream, a);
+    hipLaunchKernelGGL((attn_fwd_bf16_kernel<4, 64, 2, 3, true>), grid, dim3(256), 0, stream, a);
   return hipGetLastError();
 }
 

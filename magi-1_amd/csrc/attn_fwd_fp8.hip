@@ -29,10 +29,7 @@ constexpr float P_SHIFT = 8.f;
 
 // FASTP (with POW2): the probabilities come from a piecewise-linear exp2 built on the matrix pipe's scaling
 // instead of the quarter-rate v_exp_f32: the score registers hold e4m3 codes (see the softmax below).
-// WHATIF (tuning builds only, timing only: the results are wrong): parts of the tile loop left out, to measure what each
-// costs.  1: no row maximum, 2: no conversions of the scores, 4: V^T fragments by two plain 16-byte reads (what a V
-// cache stored in blocks of 16 keys would allow), 16: no barrier and no wait for the tile.
-template <bool POW2, bool FASTP = false, int WHATIF = 0>
+template <bool POW2, bool FASTP = false>
 __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKernArgs a) {
   // Two (K tile, V tile) buffers as four separate objects that are only ever indexed statically: the compiler
   // then knows that a read of one buffer cannot alias the direct-to-LDS loads in flight to the other and does
@@ -213,10 +210,8 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       pe1 = (k1 < ke) ? piece_end(k1, chunk1) : ke;
       new_piece1 = true;
     }
-    if constexpr (!(WHATIF & 16)) {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      __syncthreads();
-    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
     if (k1 < ke) issue_tile(k1, pe1, std::integral_constant<int, BUF ^ 1>{});
     if (wave_on) {
       const unsigned char* const Kt = BUF ? sK1 : sK0;
@@ -241,12 +236,6 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       };
       auto read_v = [&](int mb) -> i32x8 {
-        if constexpr (WHATIF & 4) {
-          const int o4 = ((l & 31) + 32 * mb) * 16 + (l >> 5) * 2048;
-          const i32x4 lo = *LDS_PTR(const i32x4, Vt + o4);
-          const i32x4 hi = *LDS_PTR(const i32x4, Vt + o4 + 4096);
-          return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
-        }
         const int o = base_v ^ (mb << 5);
         i32x2 r[4];
 #pragma unroll
@@ -301,13 +290,11 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           }
       }
       float mx = max3(s_acc[0][0], s_acc[0][1], s_acc[0][2]);
-      if constexpr (!(WHATIF & 1)) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-          for (int v = (t == 0 ? 3 : 0); v < 16; v += 2) mx = max3(mx, s_acc[t][v], s_acc[t][v + 1 < 16 ? v + 1 : v]);
-        mx = half_swap_max(mx);
-      }
+        for (int v = (t == 0 ? 3 : 0); v < 16; v += 2) mx = max3(mx, s_acc[t][v], s_acc[t][v + 1 < 16 ? v + 1 : v]);
+      mx = half_swap_max(mx);
       if constexpr (POW2) {
         // s_acc already holds exponent - m_run + shift; a value above `shift` is a new row maximum
         const float over = mx - (shift * XS + XB);
@@ -337,9 +324,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         for (int n = 0; n < 8; ++n) {  // dword n = slots 4n .. 4n+3 = s_acc[n >> 2][4 (n & 3) .. +3]
           const float x0 = s_acc[n >> 2][4 * (n & 3) + 0], x1 = s_acc[n >> 2][4 * (n & 3) + 1];
           const float x2 = s_acc[n >> 2][4 * (n & 3) + 2], x3 = s_acc[n >> 2][4 * (n & 3) + 3];
-          if constexpr (FASTP && (WHATIF & 2)) {
-            pb[n] = __builtin_bit_cast(int, x0) ^ __builtin_bit_cast(int, x3);
-          } else if constexpr (FASTP) {  // (the conversion saturates at 0 for negative values and -inf: a probability of 0)
+          if constexpr (FASTP) {  // (the conversion saturates at 0 for negative values and -inf: a probability of 0)
             unsigned u = __builtin_amdgcn_cvt_pk_u8_f32(x0, 0, 0u);
             u = __builtin_amdgcn_cvt_pk_u8_f32(x1, 1, u);
             u = __builtin_amdgcn_cvt_pk_u8_f32(x2, 2, u);
@@ -597,26 +582,6 @@ __global__ __launch_bounds__(QT1) void quantize_groups_kernel(const char* x, lon
 
 hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream) {
   const unsigned grid = a.per_xcd * 8u;
-#ifdef MAGI_TUNING
-  // MAGI_ATTN_LDS_PAD = bytes of unused dynamic LDS per workgroup: 24576 leaves two workgroups per CU, 65536 one
-  static const int lds_pad = [] { const char* e = getenv("MAGI_ATTN_LDS_PAD"); return e ? atoi(e) : 0; }();
-  if (lds_pad > 0 && (a.flags & 1) && (a.flags & 4) && a.variant == 0) {
-    (void)hipFuncSetAttribute((const void*)attn_fwd_fp8_kernel<true, true>, hipFuncAttributeMaxDynamicSharedMemorySize, lds_pad);
-    hipLaunchKernelGGL((attn_fwd_fp8_kernel<true, true>), dim3(grid), dim3(64 * NW), lds_pad, stream, a);
-    return hipGetLastError();
-  }
-#endif
-#ifdef MAGI_TUNING
-#define MAGI_WHATIF_CASE(W)                                                                                   \
-  case 100 + W:                                                                                               \
-    hipLaunchKernelGGL((attn_fwd_fp8_kernel<true, true, W>), dim3(grid), dim3(64 * NW), 0, stream, a);        \
-    return hipGetLastError();
-  if ((a.flags & 1) && (a.flags & 4)) switch (a.variant) {  // MAGI_ATTN_VARIANT = 100 + WHATIF
-      MAGI_WHATIF_CASE(1) MAGI_WHATIF_CASE(2) MAGI_WHATIF_CASE(3) MAGI_WHATIF_CASE(4) MAGI_WHATIF_CASE(16)
-      default: break;
-    }
-#undef MAGI_WHATIF_CASE
-#endif
   if ((a.flags & 1) && (a.flags & 4))
     hipLaunchKernelGGL((attn_fwd_fp8_kernel<true, true>), dim3(grid), dim3(64 * NW), 0, stream, a);
   else if (a.flags & 1)

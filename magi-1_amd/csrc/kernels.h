@@ -30,11 +30,10 @@ struct AttnKernArgs {
   int total_q, total_k, k_split;
   int n_ranges, ranges_mode, tiles_per_range;
   int block_m;  // q rows per workgroup (the launchers map it to an instantiation)
-  int variant;  // tuning builds: bf16 kernel instantiation picked by hand (0 = the library's own choice)
   int Hq, Hkv, G;
   int scale_chunk_tokens;
   int scale_split_chunk;  // first chunk served by the side segment's scale tables (INT_MAX without them)
-  int flags;  // MAGI_ATTN_* bits of the public header, plus ATTN_BOUNDED
+  int flags;  // MAGI_ATTN_* bits of the public header, plus ATTN_BOUNDED / ATTN_SCALE_Q
   unsigned total_wgs, per_xcd;
   float scale_log2;  // softmax_scale * log2(e)
   float q_norm_eps;
@@ -44,6 +43,8 @@ struct AttnKernArgs {
 
 // internal flag: the caller promised bounded scores (magi_attn_args.score_bound within MAGI_SCORE_BOUND_MAX)
 constexpr int ATTN_BOUNDED = 1 << 8;
+// internal flag (with ATTN_BOUNDED): q is unscaled, the kernel multiplies it by scale_log2 while loading it
+constexpr int ATTN_SCALE_Q = 1 << 9;
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream);
 hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream);
@@ -96,7 +97,6 @@ struct QkvGemmKernArgs {
   int batch;
   float q_premul;
   int n_row_tiles, n_col_tiles;  // filled by the launcher
-  int variant;                   // 4: the 4-wavefront form (tuning builds)
 };
 hipError_t launch_qkv_gemm_prologue(const QkvGemmKernArgs& a, hipStream_t stream);
 

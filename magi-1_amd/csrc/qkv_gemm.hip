@@ -319,19 +319,11 @@ hipError_t launch_qkv_gemm_prologue(const QkvGemmKernArgs& a_in, hipStream_t str
   a.n_row_tiles = (a.S + BM - 1) / BM;
   a.n_col_tiles = (a.Hq + 2 * a.Hkv + a.Hqx) / 2;
   const int lds = 4 * TILE + 1024;  // 129 KB of the CU's 160: above the default limit, asked for per launch (a host-side setting)
-#ifdef MAGI_TUNING
-  if (const char* v = getenv("MAGI_GEMM_WAVES")) a.variant = atoi(v);
-#endif
-  const bool four = a.variant == 4;  // (8 wavefronts of 128 x 64 unless a tuning build asks for 4 of 128 x 128)
-  const void* fn = four ? (const void*)qkv_gemm_prologue_kernel<4> : (const void*)qkv_gemm_prologue_kernel<2>;
-  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+  hipError_t e = hipFuncSetAttribute((const void*)qkv_gemm_prologue_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return e;
   const int supers = (a.n_row_tiles + 63) / 64;
   const unsigned grid = (unsigned)supers * 8u * 8u * (unsigned)a.n_col_tiles;
-  if (four)
-    hipLaunchKernelGGL(qkv_gemm_prologue_kernel<4>, dim3(grid), dim3(256), lds, stream, a);
-  else
-    hipLaunchKernelGGL(qkv_gemm_prologue_kernel<2>, dim3(grid), dim3(512), lds, stream, a);
+  hipLaunchKernelGGL(qkv_gemm_prologue_kernel<2>, dim3(grid), dim3(512), lds, stream, a);
   return hipGetLastError();
 }
 

@@ -9,9 +9,7 @@ import ctypes as C
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-# MAGI_ATTN_LIBRARY names another build of the same library (e.g. a measurement build made with `make TUNING=1 OUT=...`);
-# it must exist: a wrong path raises like a missing library does
-LIB_PATH = os.environ.get("MAGI_ATTN_LIBRARY") or os.path.join(_HERE, "libmagi_attn.so")
+LIB_PATH = os.path.join(_HERE, "libmagi_attn.so")
 
 MAGI_DTYPE_BF16 = 0
 MAGI_DTYPE_FP8_E4M3 = 1

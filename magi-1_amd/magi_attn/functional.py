@@ -91,7 +91,9 @@ def range_attention(
     q_prescaled (bf16): q already carries softmax_scale * log2(e) (qk_prologue(..., q_premul=that)), so q . k is the
     exp2 exponent: the kernel skips its per-score multiply; softmax_scale is ignored.
 
-    score_bound (with q_prescaled): promise that |q . k| <= score_bound for every pair; see magi_attn_args.score_bound.
+    score_bound: promise that |q . k| * softmax_scale * log2(e) <= score_bound for every pair (with q_prescaled the
+    factor is already in q); see magi_attn_args.score_bound.  Without q_prescaled the kernel applies the scale while
+    it loads q.
     q_tile_rows: force a workgroup shape (0 = the library's choice); see magi_attn_args.q_tile_rows.
     q_norm: (gamma, beta or None, eps[, norm_kind]): q is the raw projection, normalised per (token, head) row inside
     the kernel (fp32, zero-centred gamma) and scaled by softmax_scale * log2(e); needs score_bound.
@@ -172,15 +174,32 @@ def range_attention(
     return out, lse
 
 
+def qk_norm_score_bound(q_norm_bound: float, k_norm_bound: float, head_dim: int = 128,
+                        softmax_scale: Optional[float] = None) -> float:
+    """score_bound for QK-normed attention from the lengths the two norms can produce (each at most
+    sqrt(head_dim) max|gamma + 1| + |beta|, which a rotary embedding preserves): Cauchy-Schwarz, in exp2-exponent
+    units, plus 1 % for the roundings to bf16."""
+    scale = head_dim ** -0.5 if softmax_scale is None else softmax_scale
+    return 1.01 * scale * math.log2(math.e) * q_norm_bound * k_norm_bound
+
+
 def flex_flash_attn_func(q, k, v, q_ranges, k_ranges, max_seqlen_q, max_seqlen_k, softmax_scale=None,
-                         deterministic=False, disable_fwd_atomic_reduction=True, **_unused):
+                         deterministic=False, disable_fwd_atomic_reduction=True, score_bound: float = 0.0, **_unused):
     """(out [Tq,Hq,D], lse [Hq,Tq]) for disjoint q ranges.  The forward has one writer per output
-    row, so it is deterministic and needs no atomic reduction whatever the two flags say."""
-    return range_attention(q, k, v, q_ranges, k_ranges, max_seqlen_q, max_seqlen_k, softmax_scale)
+    row, so it is deterministic and needs no atomic reduction whatever the two flags say.
+
+    score_bound (no counterpart in the reference's call, optional): the caller's promise that
+    |q . k| * softmax_scale * log2(e) <= score_bound for every pair, with q unscaled as the reference passes it
+    (qk_norm_score_bound derives it from the norm parameters).  Up to MAGI_SCORE_BOUND_MAX it selects the kernel
+    without a running maximum, which applies the scale while it loads q."""
+    return range_attention(q, k, v, q_ranges, k_ranges, max_seqlen_q, max_seqlen_k, softmax_scale,
+                           score_bound=score_bound)
 
 
-def flash_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, deterministic=False, **_unused):
-    """q [B,Sq,Hq,D], k/v [B,Sk,Hkv,D] -> [B,Sq,Hq,D]; non-causal, no dropout (what the reference uses)."""
+def flash_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, deterministic=False,
+                    score_bound: float = 0.0, **_unused):
+    """q [B,Sq,Hq,D], k/v [B,Sk,Hkv,D] -> [B,Sq,Hq,D]; non-causal, no dropout (what the reference uses).
+    score_bound: as in flex_flash_attn_func."""
     if dropout_p != 0.0 or causal:
         raise NotImplementedError("dropout / causal are not part of the MAGI-1 attention path")
     B, Sq, Hq, D = q.shape
@@ -191,18 +210,18 @@ def flash_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, de
     cu_q = torch.arange(0, (B + 1) * Sq, Sq, dtype=torch.int32, device=q.device)
     cu_k = torch.arange(0, (B + 1) * Sk, Sk, dtype=torch.int32, device=q.device)
     out, _ = range_attention(q3, k3, v3, cu_q, cu_k, Sq, Sk, softmax_scale, ranges_mode=L.MAGI_RANGES_CU,
-                             return_lse=False, zero_init=False)
+                             return_lse=False, zero_init=False, score_bound=score_bound)
     return out.view(B, Sq, Hq, D)
 
 
 def flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p=0.0,
-                           softmax_scale=None, causal=False, deterministic=False, **_unused):
+                           softmax_scale=None, causal=False, deterministic=False, score_bound: float = 0.0, **_unused):
     """Packed varlen attention; segment s pairs q[cu_q[s]:cu_q[s+1]] with k[cu_k[s]:cu_k[s+1]].
-    A segment without keys yields zero rows."""
+    A segment without keys yields zero rows.  score_bound: as in flex_flash_attn_func."""
     if dropout_p != 0.0 or causal:
         raise NotImplementedError("dropout / causal are not part of the MAGI-1 attention path")
     out, _ = range_attention(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale,
-                             ranges_mode=L.MAGI_RANGES_CU, return_lse=False, zero_init=True)
+                             ranges_mode=L.MAGI_RANGES_CU, return_lse=False, zero_init=True, score_bound=score_bound)
     return out
 
 

@@ -145,14 +145,70 @@ def test_bounded_cache_views_two_segments_and_grouped_output(dev):
 def test_score_bound_argument_checks(dev):
     q = torch.zeros(4, 1, 128, dtype=torch.bfloat16, device=dev)
     r = torch.tensor([[0, 4]], dtype=torch.int32, device=dev)
-    with pytest.raises(M.MagiError):  # the bound is in the units of a pre-scaled q
-        M.range_attention(q, q, q, r, r, 4, score_bound=8.0)
+    q8 = q.view(torch.uint8)[..., :128].view(torch.float8_e4m3fn)
+    one = torch.ones(1, 1, device=dev)
+    with pytest.raises(M.MagiError):  # a promise about bf16 inputs
+        M.range_attention(q8, q8, q8, r, r, 4, q_scale=one, k_scale=one, v_scale=one, scale_chunk_tokens=4, score_bound=8.0)
+    with pytest.raises(M.MagiError):  # unscaled q with a bound: 256-row workgroups only
+        M.range_attention(q, q, q, r, r, 4, score_bound=8.0, q_tile_rows=512)
     with pytest.raises(M.MagiError):
         M.range_attention(q, q, q, r, r, 4, q_prescaled=True, score_bound=-1.0)
     with pytest.raises(M.MagiError):  # 384-row workgroups belong to the online-softmax kernel
         M.range_attention(q, q, q, r, r, 4, q_prescaled=True, score_bound=8.0, q_tile_rows=384)
     with pytest.raises(M.MagiError):
         M.range_attention(q, q, q, r, r, 4, q_tile_rows=512)
+
+
+@pytest.mark.parametrize("L,dn,sp,Hq,Hkv", CASES)
+def test_bound_on_unscaled_q_scales_while_loading(dev, L, dn, sp, Hq, Hkv):
+    """A score bound WITHOUT q_prescaled, as the reference-shaped callables pass it (the reference hands its
+    attention functions unscaled q and softmax_scale=None): the kernel multiplies q by softmax_scale * log2(e) while
+    loading it.  q is then rounded to bf16 twice (once by its producer, once after the scale), each 2^-9 relative
+    per element, which moves a score by ~2e-3 exp2 units r.m.s.: well inside the bf16 bar against the oracle on the
+    unscaled q, and close to the kernel fed with q pre-scaled ahead of its single rounding."""
+    q, k, v = O.synthetic_qkv(dn * L, (sp + dn) * L, Hq, Hkv, 128, seed=4321 + L)
+    bound = M.qk_norm_score_bound(q.float().norm(dim=-1).max().item(), k.float().norm(dim=-1).max().item() if k.numel() else 1.0)
+    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
+    ref = O.range_attention(q, k, v, qr, kr)
+    lse_ref = O.range_attention_lse(q, k, v, qr, kr)
+    tq, tk = _ranges(dev, qr, kr)
+    out, lse = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, int(kr.max() - kr.min()),
+                                      score_bound=bound)
+    _cmp(out, ref, f"L={L}")
+    assert (lse.cpu() - lse_ref).abs().max() < 5e-3
+    online, _ = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, int(kr.max() - kr.min()))
+    assert (out.float() - online.float()).abs().max().item() <= 2e-2
+    # an explicit softmax_scale is honoured (the bound is stated in the units of the scaled scores)
+    out2, _ = M.flex_flash_attn_func(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, int(kr.max() - kr.min()),
+                                     softmax_scale=0.05, score_bound=bound)
+    _cmp(out2, O.range_attention(q, k, v, qr, kr, softmax_scale=0.05), f"L={L} scale 0.05")
+
+
+def test_reference_shaped_callables_take_a_score_bound(dev):
+    """flash_attn_func / flash_attn_varlen_func with score_bound=: batched and varlen forms, an empty segment, the
+    interleaved cache read in place: same results as without the bound, to the rounding of the probabilities."""
+    g = torch.Generator().manual_seed(9)
+    B, Sq, Sk, Hq, Hkv, D = 3, 70, 150, 4, 2, 128
+    q = O.rmsnorm(torch.randn(B, Sq, Hq, D, generator=g)).bfloat16()
+    k = O.rmsnorm(torch.randn(B, Sk, Hkv, D, generator=g)).bfloat16()
+    v = torch.randn(B, Sk, Hkv, D, generator=g).bfloat16()
+    bound = M.qk_norm_score_bound(1.01 * D ** 0.5, 1.01 * D ** 0.5)
+    out = M.flash_attn_func(q.to(dev), k.to(dev), v.to(dev), score_bound=bound)
+    for b in range(B):
+        _cmp(out[b], O.range_attention(q[b], k[b], v[b], [[0, Sq]], [[0, Sk]]), f"batch {b}")
+    Lq = 130
+    lens = [800, 0, 20, 413]
+    qx = O.rmsnorm(torch.randn(len(lens) * Lq, Hq, D, generator=g)).bfloat16()
+    kvx = torch.randn(sum(lens), Hkv, 2 * D, generator=g)
+    kvx[..., :D] = O.rmsnorm(kvx[..., :D])
+    kvx = kvx.bfloat16()
+    cu_q = torch.arange(0, (len(lens) + 1) * Lq, Lq, dtype=torch.int32)
+    cu_k = torch.tensor(np.cumsum([0] + lens), dtype=torch.int32)
+    kd = kvx.to(dev)
+    ox = M.flash_attn_varlen_func(qx.to(dev), kd[..., :D], kd[..., D:], cu_q.to(dev), cu_k.to(dev), Lq, 800,
+                                  score_bound=bound)
+    assert torch.all(ox[Lq:2 * Lq] == 0)
+    _cmp(ox, O.varlen_cross_attention(qx, kvx[..., :D], kvx[..., D:], cu_q, cu_k))
 
 
 @pytest.mark.parametrize("kind", ["layernorm", "rmsnorm"])

@@ -195,130 +195,7 @@ def test_rejects_bad_arguments(dev):
         M.range_attention(q.float(), k, k, r, r, 8)
 
 
-# ----------------------------------------------------------------------------- full-size shapes
-def _full_size_check(dev, L, dn, sp, Hq, Hkv, seed, rows_per_chunk, cpu_rows):
-    """Benchmark-size run checked on a row subsample (rows are independent, so the subsample is
-    exact): fp32 on the GPU with plain matmuls for many rows, the CPU oracle for a few."""
-    D = 128
-    g = torch.Generator(device=dev).manual_seed(seed)
-    q = torch.randn(dn * L, Hq, D, device=dev, generator=g)
-    q = (q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
-    cache = torch.randn((sp + dn) * L, Hkv, 2 * D, device=dev, generator=g)
-    kf = cache[..., :D]
-    cache[..., :D] = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + 1e-6)
-    cache = cache.bfloat16()
-    qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
-    tq, tk = _ranges(dev, qr, kr)
-    out, lse = M.range_attention(q, cache[..., :D], cache[..., D:], tq, tk, L)
-    torch.cuda.synchronize()
-    assert torch.isfinite(out).all()
-    G = Hq // Hkv
-    rs = np.random.default_rng(seed)
-    for i in range(dn):
-        rows = torch.tensor(np.sort(rs.choice(L, rows_per_chunk, replace=False)) + i * L, device=dev)
-        ke = int(kr[i, 1])
-        qs = q[rows].float()  # [r, Hq, D]
-        ref = torch.empty(rows_per_chunk, Hq, D, device=dev)
-        for hk in range(Hkv):
-            kk, vv = cache[:ke, hk, :D].float(), cache[:ke, hk, D:].float()
-            s = torch.einsum("rgd,kd->rgk", qs[:, hk * G:(hk + 1) * G], kk) * D ** -0.5
-            ref[:, hk * G:(hk + 1) * G] = torch.einsum("rgk,kd->rgd", torch.softmax(s, -1), vv)
-        _cmp(out[rows], ref, f"chunk {i} GPU fp32 subsample")
-        # a few of those rows through the CPU oracle as well
-        sub = rows[:cpu_rows].cpu()
-        o_cpu = O.range_attention(q[sub].cpu(), cache[:ke, :, :D].cpu(), cache[:ke, :, D:].cpu(), [[0, cpu_rows]], [[0, ke]])
-        _cmp(out[sub], o_cpu, f"chunk {i} CPU oracle subsample")
-        assert (ref[:cpu_rows].cpu() - o_cpu).abs().max() < 1e-4
-    # size-independent property: values all ones -> output all ones
-    ones = cache.clone()
-    ones[..., D:] = 1
-    o1, _ = M.range_attention(q, ones[..., :D], ones[..., D:], tq, tk, L, return_lse=False)
-    assert (o1.float() - 1).abs().max() <= 2 ** -7
-    del ones, o1
-    # the pre-scaled path (q carries softmax_scale * log2(e)) at the same size, on the last chunk's subsample
-    import math
-    qp = (q.float() * (D ** -0.5 * math.log2(math.e))).bfloat16()
-    outp, _ = M.range_attention(qp, cache[..., :D], cache[..., D:], tq, tk, L, q_prescaled=True, return_lse=False)
-    i = dn - 1
-    rows = torch.tensor(np.sort(rs.choice(L, rows_per_chunk, replace=False)) + i * L, device=dev)
-    ke = int(kr[i, 1])
-    ref = torch.empty(rows_per_chunk, Hq, D, device=dev)
-    for hk in range(Hkv):
-        kk, vv = cache[:ke, hk, :D].float(), cache[:ke, hk, D:].float()
-        s2 = torch.einsum("rgd,kd->rgk", qp[rows][:, hk * G:(hk + 1) * G].float(), kk) * math.log(2.0)
-        ref[:, hk * G:(hk + 1) * G] = torch.einsum("rgk,kd->rgd", torch.softmax(s2, -1), vv)
-    _cmp(outp[rows], ref, "pre-scaled q, GPU fp32 subsample")
-
-
-def test_full_size_480p_layer(dev):
-    _full_size_check(dev, 9360, 4, 4, 24, 8, seed=2234, rows_per_chunk=256, cpu_rows=8)
-
-
-def test_full_size_720p_layer(dev):
-    _full_size_check(dev, 21600, 4, 8, 48, 8, seed=3234, rows_per_chunk=128, cpu_rows=4)
-
-
-def test_full_size_ragged_batch_with_cross_attention(dev):
-    """Four videos packed on one token axis with 1, 2, 3 and 4 active 9360-token chunks and 0-6 cached prefix chunks
-    each (seeded), chunk-causal inside each video (24 / 8 heads), then cross attention from every video token to that
-    video's T5 tokens (valid lengths uniform 20-800, K / V on 24 heads).  Checked on row subsamples: fp32 matmuls on
-    the GPU, a few rows through the CPU oracle; V = 1 gives O = 1 on every covered row."""
-    L, Hq, Hkv, D = 9360, 24, 8, 128
-    rs = np.random.default_rng(5234)
-    active = [1, 2, 3, 4]
-    prefix = [int(x) for x in rs.integers(0, 7, size=4)]
-    lens = [int(x) for x in rs.integers(20, 801, size=4)]
-    qr, kr, seg_len = [], [], []
-    qpos = kbase = 0
-    for a, p, n in zip(active, prefix, lens):
-        for j in range(a):
-            qr.append([qpos, qpos + L])
-            kr.append([kbase, kbase + (p + j + 1) * L])
-            seg_len.append(n)  # every chunk of a video attends to that video's caption
-            qpos += L
-        kbase += (p + a) * L
-    Tq, Tk = qpos, kbase
-    g = torch.Generator(device=dev).manual_seed(5234)
-    q = torch.randn(Tq, Hq, D, device=dev, generator=g)
-    q = (q * torch.rsqrt(q.pow(2).mean(-1, keepdim=True) + 1e-6)).bfloat16()
-    cache = torch.randn(Tk, Hkv, 2 * D, device=dev, generator=g)
-    kf = cache[..., :D]
-    cache[..., :D] = kf * torch.rsqrt(kf.pow(2).mean(-1, keepdim=True) + 1e-6)
-    cache = cache.bfloat16()
-    tq, tk = _ranges(dev, qr, kr)
-    out, _ = M.range_attention(q, cache[..., :D], cache[..., D:], tq, tk, L, return_lse=False)
-    G = Hq // Hkv
-    for i, ((q0, _), (k0, k1)) in enumerate(zip(qr, kr)):
-        rows = torch.tensor(np.sort(rs.choice(L, 64, replace=False)) + q0, device=dev)
-        qs = q[rows].float()
-        ref = torch.empty(64, Hq, D, device=dev)
-        for hk in range(Hkv):
-            kk, vv = cache[k0:k1, hk, :D].float(), cache[k0:k1, hk, D:].float()
-            sc = torch.einsum("rgd,kd->rgk", qs[:, hk * G:(hk + 1) * G], kk) * D ** -0.5
-            ref[:, hk * G:(hk + 1) * G] = torch.einsum("rgk,kd->rgd", torch.softmax(sc, -1), vv)
-        _cmp(out[rows], ref, f"self range {i} GPU fp32 subsample")
-        sub = rows[:4].cpu()
-        o_cpu = O.range_attention(q[sub].cpu(), cache[k0:k1, :, :D].cpu(), cache[k0:k1, :, D:].cpu(), [[0, 4]],
-                                  [[0, k1 - k0]])
-        _cmp(out[sub], o_cpu, f"self range {i} CPU oracle subsample")
-    ones = cache.clone()
-    ones[..., D:] = 1
-    o1, _ = M.range_attention(q, ones[..., :D], ones[..., D:], tq, tk, L, return_lse=False)
-    assert (o1.float() - 1).abs().max() <= 2 ** -7
-    # cross attention: one segment per chunk, L queries against its video's caption
-    cu_q = torch.arange(0, Tq + 1, L, dtype=torch.int32, device=dev)
-    cu_k = torch.tensor(np.concatenate([[0], np.cumsum(seg_len)]), dtype=torch.int32, device=dev)
-    kvx = torch.randn(int(cu_k[-1]), Hq, 2 * D, device=dev, generator=g).bfloat16()
-    xo = M.flash_attn_varlen_func(q, kvx[..., :D], kvx[..., D:], cu_q, cu_k, L, 800)
-    for i, n in enumerate(seg_len):
-        rows = torch.tensor(np.sort(rs.choice(L, 64, replace=False)) + i * L, device=dev)
-        k0 = int(cu_k[i])
-        sc = torch.einsum("rhd,khd->rhk", q[rows].float(), kvx[k0:k0 + n, :, :D].float()) * D ** -0.5
-        ref = torch.einsum("rhk,khd->rhd", torch.softmax(sc, -1), kvx[k0:k0 + n, :, D:].float())
-        _cmp(xo[rows], ref, f"cross segment {i} GPU fp32 subsample")
-        sub = rows[:4].cpu()
-        o_cpu = O.range_attention(q[sub].cpu(), kvx[k0:k0 + n, :, :D].cpu(), kvx[k0:k0 + n, :, D:].cpu(), [[0, 4]], [[0, n]])
-        _cmp(xo[sub], o_cpu, f"cross segment {i} CPU oracle subsample")
+# (the benchmark-size shapes are in tests/test_full_size_gpu.py, for every shipped kernel instantiation)
 
 
 def test_grouped_output_layout(dev):

@@ -30,20 +30,25 @@ def test_library_loads_and_exports_every_declared_symbol():
 
 
 def test_missing_library_is_an_error_not_a_fallback(tmp_path):
-    """The library named by MAGI_ATTN_LIBRARY is the one that is loaded; when it does not exist the first call
-    raises (there is no other compute path to fall back to)."""
+    """The library beside the package is the only compute path: when it is not there the first call raises (checked
+    in a child process on a copy of the package without its .so; no environment variable redirects the loader)."""
+    import shutil
     import subprocess
     import sys
 
+    pkg = tmp_path / "magi_attn"
+    shutil.copytree(os.path.join(ROOT, "magi-1_amd", "magi_attn"), pkg,
+                    ignore=shutil.ignore_patterns("*.so", "__pycache__"))
     code = (
-        "import sys; sys.path.insert(0, %r); sys.path.insert(0, %r)\n"
+        "import sys; sys.path.insert(0, %r)\n"
         "import magi_attn._lib as L\n"
+        "assert L.LIB_PATH.startswith(%r), L.LIB_PATH\n"
         "try:\n"
         "    L.lib()\n"
         "except RuntimeError as e:\n"
         "    assert 'no fallback' in str(e), e; print('raised')\n"
-    ) % (os.path.join(ROOT, "magi-1_amd"), ROOT)
-    env = dict(os.environ, MAGI_ATTN_LIBRARY=str(tmp_path / "absent" / "libmagi_attn.so"))
+    ) % (str(tmp_path), str(pkg))
+    env = dict(os.environ, MAGI_ATTN_LIBRARY=os.path.join(ROOT, "magi-1_amd", "magi_attn", "libmagi_attn.so"))
     r = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, timeout=300)
     assert r.returncode == 0 and r.stdout.strip() == "raised", (r.stdout, r.stderr[-2000:])
 
@@ -270,7 +275,7 @@ def test_attention_kernels_keep_their_registers():
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
              "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage", "-c", "-o", os.devnull]
     # the 64-row kernel: no scratch at all in the plain instantiations; the one that normalises q while loading it
-    # (template arguments <..., false, true, 0>, mangled ...ELb0ELb1ELi0EE) may park values around that prologue, outside the loop
+    # (last template argument QMODE = 1, mangled ...ELi4ELi1EE) may park values around that prologue, outside the loop
     for src, limit in (("attn_fwd_bf16.hip", 0), ("attn_fwd_fp8.hip", 24), ("attn_fwd_bf16_w64.hip", 0)):
         r = subprocess.run([hipcc] + flags + [os.path.join(csrc, src)], capture_output=True, text=True, timeout=600)
         assert r.returncode == 0, r.stderr[-2000:]
@@ -282,7 +287,7 @@ def test_attention_kernels_keep_their_registers():
         for n, sc, vg in zip(names, scratch, vgprs):
             if "attn_fwd" in n:
                 seen += 1
-                lim = 128 if (src == "attn_fwd_bf16_w64.hip" and n.endswith("ELb0ELb1ELi0EEEvNS_12AttnKernArgsE")) else limit
+                lim = 128 if (src == "attn_fwd_bf16_w64.hip" and n.endswith("ELi4ELi1EEEvNS_12AttnKernArgsE")) else limit
                 assert sc <= lim, f"{n}: {sc} bytes of scratch per lane"
                 assert vg <= 256
         assert seen >= 2

@@ -40,7 +40,9 @@ extern "C" {
  * score instead of the quarter-rate exponential this kernel is otherwise bound by.  At most 6.2 % above 2^e; the
  * row sums are taken from the same values, so the average excess cancels in the normalisation and a relative
  * spread of 2 % per weight remains, to be compared with the 2.7 % r.m.s. of rounding the probabilities to e4m3,
- * which both variants do.  lse is biased by up to +0.06 (natural log units). */
+ * which both variants do.  lse is biased by up to +0.06 (natural log units).  An opt-in approximation: the modes
+ * WITHOUT this flag evaluate the exponential exactly in fp32 ("softmax in fp32" of the fp8 benchmark configuration)
+ * and are what FullyParallelAttention(attention_dtype="fp8") runs by default. */
 #define MAGI_ATTN_FP8_FAST_EXP2 4
 /* bf16 path: q already carries softmax_scale * log2(e) (magi_qk_prologue with q_premul set to it multiplies before
  * its one rounding to bf16, so nothing is lost), i.e. the scores q.k are exp2 exponents.  The kernel then skips the
@@ -56,8 +58,14 @@ extern "C" {
 #define MAGI_NORM_RMSNORM_1P 1   /* x/sqrt(mean(x^2)+eps) * (gamma+1)          */
 #define MAGI_NORM_NONE 2
 
+/* 100 * major + minor.  The layout of the argument structs below belongs to the version; every struct also starts
+ * with its own size as the caller compiled it (struct_size = sizeof(the struct)), and an entry point that is handed
+ * another size returns MAGI_EINVAL instead of reading fields the caller never wrote. */
 int magi_version(void);
 const char* magi_last_error(void);
+/* Diagnostics: the number of kernel launches the library has issued in this process so far (all threads, all
+ * entry points).  A caller can difference it around a piece of work to see how many launches that work costs. */
+uint64_t magi_launch_count(void);
 
 /*
  * Range attention forward (bf16 or fp8-e4m3 inputs, fp32 softmax, bf16 output).
@@ -89,7 +97,12 @@ const char* magi_last_error(void);
  *                        the core and the cross attention write straight into the "(hn n hd)" buffer that
  *                        linear_proj consumes, which removes the concat + rearrange of attn_linear_proj
  *                        (inference/model/dit/dit_module.py:1332-1340).
- * lse                    optional fp32 [Hq, total_q] (NULL to skip)
+ * lse                    optional fp32 [Hq, total_q] (NULL to skip): log sum exp of the scaled scores (natural log).
+ *                        bf16 kernels sum the fp32 probabilities (within 1e-3 of the fp32 value; the bounded-score
+ *                        kernel within 1e-5).  The fp8 kernel takes its row sums on the matrix pipe from the
+ *                        probabilities AFTER their rounding to e4m3 (what the P V product uses): lse is within
+ *                        2e-2 of the fp32 value in the exact-exponential modes, and up to 0.06 high with
+ *                        MAGI_ATTN_FP8_FAST_EXP2.
  * q_ranges, k_ranges     DEVICE int32 arrays, encoding per ranges_mode; clamped to
  *                        [0,total_q] / [0,total_k] in the kernel
  * max_seqlen_q           upper bound of any q range length (host int; sizes the grid: rows of a range beyond
@@ -98,15 +111,19 @@ const char* magi_last_error(void);
  * q_scale,k_scale,v_scale  fp8 only: DEVICE fp32 [n_scale_chunks, H] with the scale of token t
  *                        at [t / scale_chunk_tokens, h]; NULL for bf16
  * softmax_scale          <= 0 selects D^-0.5
- * score_bound            0 = unknown.  > 0 (bf16 with MAGI_ATTN_Q_PRESCALED only): the caller's promise that every
- *                        score satisfies |q . k| <= score_bound, in the units q was pre-scaled to (exp2 exponents).
+ * score_bound            0 = unknown.  > 0 (bf16 only): the caller's promise that every score satisfies
+ *                        |q . k| * softmax_scale * log2(e) <= score_bound, i.e. a bound on the exp2 exponents
+ *                        (with MAGI_ATTN_Q_PRESCALED the factor is already in q and the bound is on |q . k| itself).
  *                        Up to MAGI_SCORE_BOUND_MAX the softmax is then evaluated as 2^score / sum 2^score without a
  *                        running maximum (it is shift invariant, and 2^score can neither overflow nor lose its
  *                        leading terms in fp32 at such bounds): the same result with a third fewer vector
- *                        instructions, and room for kernels that hold 64 query rows per wavefront.  QK-normed
- *                        attention knows the bound from its norm parameters:
+ *                        instructions, and room for kernels that hold 64 query rows per wavefront.  Unscaled q (no
+ *                        MAGI_ATTN_Q_PRESCALED, what the reference's call sites pass) is multiplied by the scale
+ *                        while the kernel loads it and rounded to bf16 a second time (2^-9 relative per element,
+ *                        like the rounding q already carries).  QK-normed attention knows the bound from its norm
+ *                        parameters:
  *                        |q| |k| <= (sqrt(D) max|gamma_q + 1| + |beta_q|) (sqrt(D) max|gamma_k + 1| + |beta_k|),
- *                        times the pre-scale factor.  Larger bounds fall back to the running maximum.  A promise
+ *                        times the scale factor.  Larger bounds fall back to the running maximum.  A promise
  *                        that does not hold gives inf / nan or wrong rows, not a fault.  No counterpart in the
  *                        reference.
  * q_norm_gamma, q_norm_beta, q_norm_eps, q_norm_kind
@@ -119,12 +136,14 @@ const char* magi_last_error(void);
  *                        MAGI_ATTN_Q_PRESCALED (the raw q is not scaled).
  * q_tile_rows            0 = the library picks the workgroup shape from the size of the launch.  Otherwise the
  *                        number of query rows per workgroup to use: 128 or 384 (bf16), 256 or 512 (bf16 with a
- *                        score_bound in force), 128 (fp8); anything else is MAGI_EINVAL.  Results do not depend on
+ *                        score_bound in force and pre-scaled q; 256 with q_norm or unscaled q), 128 (fp8); anything
+ *                        else is MAGI_EINVAL.  Results do not depend on
  *                        it beyond the order of fp32 additions; it exists so that every shipped workgroup shape
  *                        can be exercised on small inputs.
  */
 #define MAGI_SCORE_BOUND_MAX 64.0f
 typedef struct magi_attn_args {
+  uint32_t struct_size; /* sizeof(magi_attn_args) */
   const void* q;
   const void* k;
   const void* v;
@@ -197,6 +216,7 @@ int magi_attn_fwd(const magi_attn_args* args, void* stream);
  *         touched (v_raw may be NULL): it has no a-priori bound; magi_quantize_fp8_split takes it from v_raw.
  */
 typedef struct magi_prologue_args {
+  uint32_t struct_size; /* sizeof(magi_prologue_args) */
   const void* q_raw;
   const void* k_raw;
   const void* v_raw;
@@ -238,6 +258,7 @@ int magi_qk_prologue(const magi_prologue_args* args, void* stream);
  * rope [S / batch, 96] fp32 (sin | cos) or NULL: this entry point implements rotary_dim 96 (R2 = 48) only.
  */
 typedef struct magi_qkv_proj_args {
+  uint32_t struct_size; /* sizeof(magi_qkv_proj_args) */
   const void* x;
   const void* w;
   int64_t x_stride, w_stride;
@@ -313,6 +334,7 @@ int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, voi
  * large groups and gives the same bytes.
  */
 typedef struct magi_quantize_args {
+  uint32_t struct_size; /* sizeof(magi_quantize_args) */
   const void* x;
   int64_t x_stride_t, x_stride_h;
   int32_t T, H, D, chunk_tokens;

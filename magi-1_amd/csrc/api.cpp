@@ -1,5 +1,6 @@
 // C-ABI layer of libmagi_attn: argument validation, error reporting, kernel dispatch.
 #include <hip/hip_runtime.h>
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -25,6 +26,16 @@ int hip_fail(hipError_t e, const char* what) {
   return fail(MAGI_EHIP, "%s: %s", what, hipGetErrorString(e));
 }
 
+std::atomic<uint64_t> g_launches{0};
+
+// the caller's view of an argument struct must be this library's
+template <class T>
+bool same_layout(const T* p) { return p->struct_size == sizeof(T); }
+#define MAGI_CHECK_LAYOUT(fn, p)                                                                            \
+  if (!same_layout(p))                                                                                      \
+    return fail(MAGI_EINVAL, fn ": struct_size %u, this library expects %zu (header / library version mismatch)", \
+                (unsigned)(p)->struct_size, sizeof(*(p)))
+
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // compute units of the current device (asked once per device; 256 when the query fails)
@@ -44,12 +55,15 @@ int compute_units() {
 
 extern "C" {
 
-int magi_version(void) { return 101; }
+int magi_version(void) { return 102; }
+
+uint64_t magi_launch_count(void) { return g_launches.load(std::memory_order_relaxed); }
 
 const char* magi_last_error(void) { return g_err; }
 
 int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   if (!p) return fail(MAGI_EINVAL, "magi_attn_fwd: args is NULL");
+  MAGI_CHECK_LAYOUT("magi_attn_fwd", p);
   if (p->D != 128) return fail(MAGI_ENOSYS, "magi_attn_fwd: head_dim %d not implemented (128 only)", p->D);
   if (p->dtype != MAGI_DTYPE_BF16 && p->dtype != MAGI_DTYPE_FP8_E4M3)
     return fail(MAGI_EINVAL, "magi_attn_fwd: unknown dtype %d", p->dtype);
@@ -215,11 +229,13 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   else
     e = magi::launch_attn_fwd_bf16(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_attn_fwd launch");
+  g_launches.fetch_add(1, std::memory_order_relaxed);
   return MAGI_OK;
 }
 
 int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   if (!p) return fail(MAGI_EINVAL, "magi_qk_prologue: args is NULL");
+  MAGI_CHECK_LAYOUT("magi_qk_prologue", p);
   if (p->D != 128) return fail(MAGI_ENOSYS, "magi_qk_prologue: head_dim %d not implemented (128 only)", p->D);
   if (p->S < 0 || p->Hq < 0 || p->Hkv < 0) return fail(MAGI_EINVAL, "magi_qk_prologue: negative size");
   if (p->S == 0 || p->Hq + p->Hkv == 0) return MAGI_OK;
@@ -284,11 +300,13 @@ int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   a.q_premul = p->q_premul == 0.f ? 1.f : p->q_premul;
   hipError_t e = magi::launch_prologue(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_qk_prologue launch");
+  g_launches.fetch_add(1, std::memory_order_relaxed);
   return MAGI_OK;
 }
 
 int magi_qkv_proj_prologue(const magi_qkv_proj_args* p, void* stream) {
   if (!p) return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: args is NULL");
+  MAGI_CHECK_LAYOUT("magi_qkv_proj_prologue", p);
   if (p->D != 128) return fail(MAGI_ENOSYS, "magi_qkv_proj_prologue: head_dim %d not implemented (128 only)", p->D);
   if (p->S < 0 || p->K <= 0 || p->Hq < 0 || p->Hkv < 0 || p->Hqx < 0)
     return fail(MAGI_EINVAL, "magi_qkv_proj_prologue: bad size");
@@ -351,6 +369,7 @@ int magi_qkv_proj_prologue(const magi_qkv_proj_args* p, void* stream) {
   a.q_premul = p->q_premul == 0.f ? 1.f : p->q_premul;
   hipError_t e = magi::launch_qkv_gemm_prologue(a, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_qkv_proj_prologue launch");
+  g_launches.fetch_add(1, std::memory_order_relaxed);
   return MAGI_OK;
 }
 
@@ -370,6 +389,7 @@ int magi_layer_norm(const void* x, int64_t x_stride, const void* weight, const v
                                          static_cast<char*>(y), y_stride * 2, rows, cols, eps,
                                          static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_layer_norm launch");
+  g_launches.fetch_add(1, std::memory_order_relaxed);
   return MAGI_OK;
 }
 
@@ -386,6 +406,7 @@ int magi_head_norm(const void* x, int64_t x_stride_t, int64_t x_stride_h, const 
   hipError_t e = magi::launch_head_norm(static_cast<const char*>(x), x_stride_t * 2, x_stride_h * 2, gamma, beta,
                                         static_cast<char*>(y), S, H, norm_kind, eps, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_head_norm launch");
+  g_launches.fetch_add(1, std::memory_order_relaxed);
   return MAGI_OK;
 }
 
@@ -397,11 +418,13 @@ int magi_apply_rotary(const void* x, const float* cos, const float* sin, void* y
   if (!x || !y || (R2 > 0 && (!cos || !sin))) return fail(MAGI_EINVAL, "magi_apply_rotary: NULL pointer");
   hipError_t e = magi::launch_rotary(x, cos, sin, y, B, S, H, D, R2, is_bf16, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return hip_fail(e, "magi_apply_rotary launch");
+  g_launches.fetch_add(1, std::memory_order_relaxed);
   return MAGI_OK;
 }
 
 static int quantize_impl(const magi_quantize_args* p, void* stream, bool always_one_launch) {
   if (!p) return fail(MAGI_EINVAL, "magi_quantize_fp8: args is NULL");
+  MAGI_CHECK_LAYOUT("magi_quantize_fp8", p);
   if (p->D != 128) return fail(MAGI_ENOSYS, "magi_quantize_fp8: head_dim %d not implemented (128 only)", p->D);
   if (p->T < 0 || p->H < 0 || p->chunk_tokens <= 0) return fail(MAGI_EINVAL, "magi_quantize_fp8: bad size");
   if (!(p->premul == p->premul) || p->premul == 0.f)
@@ -418,11 +441,13 @@ static int quantize_impl(const magi_quantize_args* p, void* stream, bool always_
     return fail(MAGI_EINVAL, "magi_quantize_fp8: y2 / scales2 needed for rows >= n_rows_first");
   if (p->x_stride_t % 8 || p->x_stride_h % 8 || !aligned16(p->x) || !aligned16(p->y) || !aligned16(p->y2))
     return fail(MAGI_EINVAL, "magi_quantize_fp8: rows must be 16-byte aligned");
+  int n_launches = 0;
   hipError_t e = magi::launch_quantize_fp8(static_cast<const char*>(p->x), p->x_stride_t * 2, p->x_stride_h * 2,
                                            static_cast<char*>(p->y), p->scales, p->T, p->H, p->chunk_tokens, p->premul,
                                            p->pow2_scales, p->n_rows_first, static_cast<char*>(p->y2), p->scales2,
-                                           always_one_launch, static_cast<hipStream_t>(stream));
+                                           always_one_launch, static_cast<hipStream_t>(stream), &n_launches);
   if (e != hipSuccess) return hip_fail(e, "magi_quantize_fp8 launch");
+  g_launches.fetch_add((uint64_t)n_launches, std::memory_order_relaxed);
   return MAGI_OK;
 }
 
@@ -432,6 +457,7 @@ int magi_quantize_fp8(const void* x, int64_t x_stride_t, int64_t x_stride_h, voi
                       int32_t H, int32_t D, int32_t chunk_tokens, float premul, int32_t pow2_scales, void* stream) {
   magi_quantize_args q;
   std::memset(&q, 0, sizeof(q));
+  q.struct_size = sizeof(q);
   q.x = x;
   q.x_stride_t = x_stride_t;
   q.x_stride_h = x_stride_h;

@@ -593,9 +593,10 @@ hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream) {
 
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
                                int chunk_tokens, float premul, int pow2_scales, int n_first, char* y2, float* scales2,
-                               bool one_launch, hipStream_t stream) {
+                               bool one_launch, hipStream_t stream, int* n_launches) {
   const int n_chunks = (T + chunk_tokens - 1) / chunk_tokens;
   const int n = n_chunks * H;
+  *n_launches = 0;
   if (n <= 0) return hipSuccess;
   // Unless asked for, one launch only when a group is small enough for one workgroup's two passes and there are
   // enough groups to spread over the chip (a second destination is served by that kernel alone); both paths give
@@ -608,6 +609,7 @@ hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, 
     share = max(1, min(share, min(16, min(chunk_tokens, T) / (4 * QROWS))));
     hipLaunchKernelGGL(quantize_groups_kernel, dim3(H, n_chunks, share), dim3(QT1), 0, stream, x, x_stride_t, x_stride_h, y,
                        scales, T, H, chunk_tokens, premul, pow2_scales, n_first, y2, scales2);
+    *n_launches = 1;
     return hipGetLastError();
   }
   hipLaunchKernelGGL(fill_zero_kernel, dim3((n + QT - 1) / QT), dim3(QT), 0, stream, (unsigned*)scales, n);
@@ -620,6 +622,7 @@ hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, 
   const long threads = (long)T * H * 16;
   hipLaunchKernelGGL(quantize_kernel, dim3((unsigned)((threads + QT - 1) / QT)), dim3(QT), 0, stream, x, x_stride_t,
                      x_stride_h, y, scales, T, H, chunk_tokens, premul);
+  *n_launches = 4;
   return hipGetLastError();
 }
 

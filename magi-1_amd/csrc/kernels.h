@@ -108,8 +108,9 @@ hipError_t launch_rotary(const void* x, const float* cos, const float* sin, void
                          int R2, int is_bf16, hipStream_t stream);
 // Rows below n_first go to y / scales, the rest (row index and chunk index counted from n_first, a multiple of
 // chunk_tokens) to y2 / scales2.  one_launch: always the single-launch kernel (else only where it is the faster).
+// *n_launches receives the number of kernels launched.
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
                                int chunk_tokens, float premul, int pow2_scales, int n_first, char* y2, float* scales2,
-                               bool one_launch, hipStream_t stream);
+                               bool one_launch, hipStream_t stream, int* n_launches);
 
 }  // namespace magi

@@ -32,8 +32,17 @@ class MagiError(RuntimeError):
         self.code = code
 
 
-class AttnArgs(C.Structure):
+class _SizedStructure(C.Structure):
+    """Every argument struct of the C-ABI starts with its own size (struct_size), filled in here."""
+
+    def __init__(self, *args, **kw):
+        super().__init__(*args, **kw)
+        self.struct_size = C.sizeof(type(self))
+
+
+class AttnArgs(_SizedStructure):
     _fields_ = [
+        ("struct_size", C.c_uint32),
         ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("k2", C.c_void_p), ("v2", C.c_void_p),
         ("out", C.c_void_p), ("lse", C.c_void_p), ("q_ranges", C.c_void_p), ("k_ranges", C.c_void_p),
         ("q_scale", C.c_void_p), ("k_scale", C.c_void_p), ("v_scale", C.c_void_p),
@@ -52,8 +61,9 @@ class AttnArgs(C.Structure):
     ]
 
 
-class PrologueArgs(C.Structure):
+class PrologueArgs(_SizedStructure):
     _fields_ = [
+        ("struct_size", C.c_uint32),
         ("q_raw", C.c_void_p), ("k_raw", C.c_void_p), ("v_raw", C.c_void_p), ("rope", C.c_void_p),
         ("gq", C.c_void_p), ("bq", C.c_void_p), ("gk", C.c_void_p), ("bk", C.c_void_p),
         ("q_out", C.c_void_p), ("kv_out", C.c_void_p), ("kv_tail", C.c_void_p),
@@ -66,8 +76,9 @@ class PrologueArgs(C.Structure):
     ]
 
 
-class QkvProjArgs(C.Structure):
+class QkvProjArgs(_SizedStructure):
     _fields_ = [
+        ("struct_size", C.c_uint32),
         ("x", C.c_void_p), ("w", C.c_void_p), ("x_stride", C.c_int64), ("w_stride", C.c_int64),
         ("S", C.c_int32), ("K", C.c_int32),
         ("Hq", C.c_int32), ("Hkv", C.c_int32), ("Hqx", C.c_int32), ("D", C.c_int32),
@@ -80,8 +91,9 @@ class QkvProjArgs(C.Structure):
     ]
 
 
-class QuantizeArgs(C.Structure):
+class QuantizeArgs(_SizedStructure):
     _fields_ = [
+        ("struct_size", C.c_uint32),
         ("x", C.c_void_p), ("x_stride_t", C.c_int64), ("x_stride_h", C.c_int64),
         ("T", C.c_int32), ("H", C.c_int32), ("D", C.c_int32), ("chunk_tokens", C.c_int32),
         ("premul", C.c_float), ("pow2_scales", C.c_int32),
@@ -90,7 +102,9 @@ class QuantizeArgs(C.Structure):
     ]
 
 
-EXPORTS = ("magi_version", "magi_last_error", "magi_attn_fwd", "magi_qk_prologue", "magi_head_norm",
+ABI_VERSION = 102  # magi_version() of the library these mirrors were written for
+
+EXPORTS = ("magi_version", "magi_last_error", "magi_launch_count", "magi_attn_fwd", "magi_qk_prologue", "magi_head_norm",
            "magi_apply_rotary", "magi_quantize_fp8", "magi_quantize_fp8_split", "magi_layer_norm", "magi_qkv_proj_prologue")
 
 _lib = None
@@ -106,6 +120,10 @@ def lib() -> C.CDLL:
                 "there is no fallback path")
         l = C.CDLL(LIB_PATH)
         l.magi_version.restype = C.c_int
+        if l.magi_version() != ABI_VERSION:
+            raise RuntimeError(f"{LIB_PATH} reports version {l.magi_version()}, this package binds version {ABI_VERSION}: "
+                               "rebuild the library (`make -C magi-1_amd/csrc`)")
+        l.magi_launch_count.restype = C.c_uint64
         l.magi_last_error.restype = C.c_char_p
         l.magi_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
         l.magi_attn_fwd.restype = C.c_int

@@ -140,6 +140,19 @@ def range_attention(
         if t is not None and (t.dtype != torch.float32 or not t.is_contiguous() or t.device != q.device):
             raise ValueError(f"{name} must be a contiguous fp32 tensor on q's device")
     a.k2_scale, a.v2_scale = _ptr(k2_scale), _ptr(v2_scale)
+    if q.dtype == torch.float8_e4m3fn and scale_chunk_tokens > 0:
+        # the kernel indexes the tables by token / scale_chunk_tokens without a bound of its own
+        C_ = int(scale_chunk_tokens)
+        rows_of = lambda n: (n + C_ - 1) // C_
+        first = total_k if (k2 is None or k2_scale is None) else int(k_split)
+        need = [("q_scale", q_scale, rows_of(Tq), Hq), ("k_scale", k_scale, rows_of(first), Hkv),
+                ("v_scale", v_scale, rows_of(first), Hkv)]
+        if k2_scale is not None:
+            need += [("k2_scale", k2_scale, rows_of(total_k - int(k_split)), Hkv),
+                     ("v2_scale", v2_scale, rows_of(total_k - int(k_split)), Hkv)]
+        for name, t, rows, heads in need:
+            if t is not None and (t.dim() != 2 or t.shape[0] < rows or t.shape[1] != heads):
+                raise ValueError(f"{name} must be [>= {rows} chunks, {heads} heads], got {tuple(t.shape)}")
     a.q_stride_t, a.q_stride_h = q.stride(0), q.stride(1)
     a.k_stride_t, a.k_stride_h = k.stride(0), k.stride(1)
     a.v_stride_t, a.v_stride_h = v.stride(0), v.stride(1)

@@ -74,7 +74,14 @@ class FusedLayerNorm(torch.nn.Module):
             g = ((w + 1).float() - 1.0) if self.zero_centered_gamma else (w.float() - 1.0)
             self.__dict__["_gb"] = (g.contiguous(), self.bias.detach().float().contiguous())
             self.__dict__["_gb_key"] = key
+            self.__dict__["_gb_epoch"] = self.__dict__.get("_gb_epoch", 0) + 1
         return self.__dict__["_gb"]
+
+    def parameter_epoch(self) -> int:
+        """A counter that advances whenever gamma_beta_fp32() had to convert the parameters anew: what values derived
+        from the parameters (score bounds, quantisation scales) key their own caches on."""
+        self.gamma_beta_fp32()
+        return self.__dict__["_gb_epoch"]
 
     def invalidate_cached_parameters(self) -> None:
         self.__dict__.pop("_gb_key", None)
@@ -91,6 +98,39 @@ class FusedLayerNorm(torch.nn.Module):
         shape = x.shape
         y = head_norm(x.reshape(-1, shape[-2], shape[-1]).to(torch.bfloat16), g, b, self.eps)
         return y.reshape(shape).to(x.dtype)
+
+
+def qk_score_bound(q_norm: FusedLayerNorm, k_norm: FusedLayerNorm, rotary_half: int = 0) -> float:
+    """Upper bound of |q . k| over all rows the two norms can produce, with a rotary embedding of 2 * rotary_half
+    features (pairs (i, i + rotary_half); 0 = none) applied to both.
+
+    A normed row is n * (gamma + 1) + beta with |n|^2 <= D.  The rotation acts inside each pair and preserves the
+    pair's length, so with groups p = the rotary pairs and the unpaired features one by one,
+    G_p = max over the group of |gamma + 1| and B_p = the length of beta inside the group:
+
+        |q . k| <= sum_p (Gq_p |nq_p| + Bq_p) (Gk_p |nk_p| + Bk_p)
+                <= D max_p(Gq_p Gk_p) + sqrt(D) (|Gq * Bk| + |Gk * Bq|) + Bq . Bk          (Cauchy-Schwarz)
+
+    which is never above the product of the two rows' lengths (sqrt(D) max|gamma + 1| + |beta|)^2 and is tighter
+    when the large gains of the two norms sit on different features.  One host read of the parameters."""
+    gq, bq = q_norm.gamma_beta_fp32()
+    gk, bk = k_norm.gamma_beta_fp32()
+    D = gq.numel()
+    r = int(rotary_half)
+    if not 0 <= 2 * r <= D:
+        raise ValueError("rotary_half must satisfy 0 <= 2 * rotary_half <= head_dim")
+
+    def groups(g, b):
+        G, B2 = (g.double() + 1.0).abs(), b.double() ** 2
+        if r:
+            Gp, Bp = torch.maximum(G[:r], G[r:2 * r]), B2[:r] + B2[r:2 * r]
+            G, B2 = torch.cat([Gp, G[2 * r:]]), torch.cat([Bp, B2[2 * r:]])
+        return G, B2.sqrt()
+
+    Gq, Bq = groups(gq, bq)
+    Gk, Bk = groups(gk, bk)
+    bound = (D * (Gq * Gk).max() + math.sqrt(D) * ((Gq * Bk).norm() + (Gk * Bq).norm()) + (Bq * Bk).sum())
+    return float(bound.item())
 
 
 class CustomLayerNormLinear(torch.nn.Module):
@@ -171,12 +211,13 @@ class FullyParallelAttention(torch.nn.Module):
     def __init__(self, hidden_size: int, num_attention_heads: int, num_query_groups: int, kv_channels: int = 128,
                  layer_number: int = 0, layernorm_epsilon: float = 1e-6, apply_layernorm_1p: bool = True,
                  xattn_cond_hidden_ratio: float = 1.0, params_dtype=torch.bfloat16, device=None,
-                 attention_dtype: str = "bf16", fp8_fast_exp2: bool = True, fused_projection: bool = False):
+                 attention_dtype: str = "bf16", fp8_fast_exp2: bool = False, fused_projection: bool = False):
         """attention_dtype "fp8" (not in the reference, which has no fp8 attention) runs the self-attention on
         e4m3 operands with per-(video chunk, head) power-of-two scales and keeps the KV cache in that form
         (Fp8KVCache); the cross attention and everything else stay in bf16.
-        fp8_fast_exp2: the fp8 kernel's piecewise-linear exp2 (MAGI_ATTN_FP8_FAST_EXP2: about 10 % faster, the
-        output within the same accuracy bar as with the exact exponential); False for the exact one.
+        fp8_fast_exp2: False (default) = the exact exponential, "softmax in fp32"; True opts into the fp8 kernel's
+        piecewise-linear exp2 (MAGI_ATTN_FP8_FAST_EXP2: about 15 % faster, probabilities up to 6.2 % off each, the
+        output inside a looser accuracy bar; see include/magi_attn.h).
         fused_projection: run the four projections and the prologue as ONE launch (magi_qkv_proj_prologue, the
         hand-written GEMM whose epilogue is the prologue) instead of a library GEMM followed by the prologue kernel;
         bf16 attention at batch 1 only.  Off by default: at the 720p shape the library GEMM + prologue take
@@ -212,20 +253,32 @@ class FullyParallelAttention(torch.nn.Module):
         self.k_layernorm_xattn = mk(params_dtype)
 
     # ------------------------------------------------------------------ score bounds
-    def score_bounds(self) -> Tuple[float, float]:
+    def score_bounds(self, rotary_half: int = 48) -> Tuple[float, float]:
         """(self attention, cross attention) upper bounds of |q . k| in exp2-exponent units (q carrying
-        softmax_scale * log2(e)), from the norm parameters: QK-normed rows have a known length, and the rotary
-        embedding preserves it.  Cauchy-Schwarz, plus 1 % for the roundings to bf16.  Within
+        softmax_scale * log2(e)), from the norm parameters (qk_score_bound: QK-normed rows have a known length, and
+        the rotary embedding of 2 * rotary_half features preserves it), plus 1 % for the roundings to bf16.  Within
         MAGI_SCORE_BOUND_MAX the attention kernels then need no running maximum (magi_attn_args.score_bound);
         larger values make them fall back to it.  Computed once per set of parameter values (it reads them on the
-        host) and cached until a parameter is modified or replaced."""
+        host) and cached until a parameter is modified or replaced (see invalidate_cached_parameters)."""
         lns = (self.q_layernorm, self.k_layernorm, self.q_layernorm_xattn, self.k_layernorm_xattn)
-        key = tuple((id(t), t._version) for ln in lns for t in (ln.weight, ln.bias))
+        key = tuple(ln.parameter_epoch() for ln in lns)
         if getattr(self, "_bounds_key", None) != key:
-            nq, nk, nqx, nkx = (ln.output_norm_bound() for ln in lns)
-            self._bounds = (1.01 * self._q_premul * nq * nk, 1.01 * self._q_premul * nqx * nkx)
-            self._bounds_key = key
-        return self._bounds
+            self._bounds, self._bounds_key = {}, key
+        r = int(rotary_half)
+        if r not in self._bounds:  # (the cross-attention half does not depend on r)
+            cross = next(iter(self._bounds.values()))[1] if self._bounds else \
+                1.01 * self._q_premul * qk_score_bound(lns[2], lns[3], 0)
+            self._bounds[r] = (1.01 * self._q_premul * qk_score_bound(lns[0], lns[1], r), cross)
+        return self._bounds[r]
+
+    def invalidate_cached_parameters(self) -> None:
+        """Forget everything derived from the norm parameters (their fp32 forms, the score bounds, the e4m3 operand
+        scales).  Needed only after a parameter was written through `.data`, which advances no version counter;
+        in-place writes (`copy_`, `load_state_dict`) and replaced parameters (`load_state_dict(assign=True)`, `.to()`)
+        are noticed by themselves."""
+        for ln in (self.q_layernorm, self.k_layernorm, self.q_layernorm_xattn, self.k_layernorm_xattn):
+            ln.invalidate_cached_parameters()
+        self._bounds_key = self._fp8_scales_key = None
 
     # ------------------------------------------------------------------ cache
     def _allocate_key_and_value_memory(self, sequence_length: int, batch_size: int, dtype) -> torch.Tensor:
@@ -259,7 +312,7 @@ class FullyParallelAttention(torch.nn.Module):
         (FusedLayerNorm.output_norm_bound) and the rotary embedding preserves, so these scales never saturate and
         the prologue can quantise without an absmax pass.  Cached like score_bounds()."""
         lns = (self.q_layernorm, self.k_layernorm)
-        key = tuple((id(t), t._version) for ln in lns for t in (ln.weight, ln.bias))
+        key = tuple(ln.parameter_epoch() for ln in lns)
         if getattr(self, "_fp8_scales_key", None) != key:
             nq, nk = (ln.output_norm_bound() for ln in lns)
             self._fp8_scales = (pow2_scale_for(self._q_premul * nq), pow2_scale_for(nk))
@@ -548,7 +601,14 @@ class FullyParallelAttention(torch.nn.Module):
         sin_emb, cos_emb = rotary_pos_emb.tensor_split(2, -1)
         # the incoming table already is the [sin | cos] layout the prologue takes
         rope = rotary_pos_emb if (rotary_pos_emb.dtype == torch.float32 and rotary_pos_emb.is_contiguous()) else None
-        bound_core = self.score_bounds()[0]
+        bound_core = self.score_bounds(rotary_pos_emb.shape[-1] // 2)[0]
+        # which attention kernels this forward selects (diagnostics; the choice follows from the norm parameters)
+        bounded = lambda b: "bounded-score, 64 rows per wavefront" if 0.0 < b <= L.MAGI_SCORE_BOUND_MAX \
+            else "online softmax, 32 rows per wavefront"
+        self.last_forward_kernels = {
+            "core": "fp8" if self.attention_dtype == "fp8" else bounded(bound_core), "core_score_bound": bound_core,
+            "cross": bounded(self.score_bounds()[1] if hidden_states.shape[1] == 1 else float("inf")),
+            "cross_score_bound": self.score_bounds()[1]}
         bs = hidden_states.shape[1]
         sq = hidden_states.shape[0]
         D = self.hidden_size_per_attention_head

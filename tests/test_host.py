@@ -57,24 +57,42 @@ def test_struct_layouts_match_header(tmp_path):
     """ctypes mirrors vs the C compiler's view of include/magi_attn.h (sizes and field offsets)."""
     import subprocess
 
-    fields_a = [f[0] for f in L.AttnArgs._fields_]
-    fields_p = [f[0] for f in L.PrologueArgs._fields_]
-    src = ['#include <stdio.h>', '#include <stddef.h>', '#include "magi_attn.h"', 'int main(void){',
-           'printf("%zu\\n", sizeof(magi_attn_args));']
-    src += ['printf("%%zu\\n", offsetof(magi_attn_args, %s));' % f for f in fields_a]
-    src += ['printf("%zu\\n", sizeof(magi_prologue_args));']
-    src += ['printf("%%zu\\n", offsetof(magi_prologue_args, %s));' % f for f in fields_p]
+    pairs = (("magi_attn_args", L.AttnArgs), ("magi_prologue_args", L.PrologueArgs),
+             ("magi_qkv_proj_args", L.QkvProjArgs), ("magi_quantize_args", L.QuantizeArgs))
+    src = ['#include <stdio.h>', '#include <stddef.h>', '#include "magi_attn.h"', 'int main(void){']
+    for cname, mirror in pairs:
+        src += ['printf("%%zu\\n", sizeof(%s));' % cname]
+        src += ['printf("%%zu\\n", offsetof(%s, %s));' % (cname, f[0]) for f in mirror._fields_]
     src += ['return 0;}']
     c = tmp_path / "layout.c"
     c.write_text("\n".join(src))
     exe = tmp_path / "layout"
     subprocess.run(["gcc", "-I", os.path.join(ROOT, "include"), str(c), "-o", str(exe)], check=True)
     out = [int(x) for x in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
-    na = len(fields_a)
-    assert out[0] == C.sizeof(L.AttnArgs)
-    assert out[1:1 + na] == [getattr(L.AttnArgs, f).offset for f in fields_a]
-    assert out[1 + na] == C.sizeof(L.PrologueArgs)
-    assert out[2 + na:] == [getattr(L.PrologueArgs, f).offset for f in fields_p]
+    pos = 0
+    for cname, mirror in pairs:
+        names = [f[0] for f in mirror._fields_]
+        assert names[0] == "struct_size" and getattr(mirror, "struct_size").offset == 0
+        assert out[pos] == C.sizeof(mirror), cname
+        assert out[pos + 1:pos + 1 + len(names)] == [getattr(mirror, f).offset for f in names], cname
+        assert mirror().struct_size == C.sizeof(mirror)  # filled in by the mirror's constructor
+        pos += 1 + len(names)
+    assert pos == len(out)
+
+
+def test_a_struct_of_another_size_is_refused():
+    """Every argument struct starts with its size as the caller compiled it; a caller built against another
+    version of the header (a shorter or longer struct) gets MAGI_EINVAL instead of having fields read that it
+    never wrote.  The Python mirrors are bound to one library version and refuse to load another."""
+    lib = magi_attn.lib()
+    assert lib.magi_version() == L.ABI_VERSION
+    for mk, fn in ((L.AttnArgs, lib.magi_attn_fwd), (L.PrologueArgs, lib.magi_qk_prologue),
+                   (L.QkvProjArgs, lib.magi_qkv_proj_prologue), (L.QuantizeArgs, lib.magi_quantize_fp8_split)):
+        a = mk()
+        for wrong in (0, a.struct_size - 8, a.struct_size + 8):
+            a.struct_size = wrong
+            assert fn(C.byref(a), None) == -22 and b"struct_size" in lib.magi_last_error(), mk.__name__
+    assert isinstance(lib.magi_launch_count(), int)
 
 
 def test_attn_argument_validation_without_gpu():

@@ -292,14 +292,114 @@ def test_layer_forward_sequence_with_kv_cache(dev):
                                          cross_p.cu_seqlens_q.cpu(), cross_p.cu_seqlens_kv.cpu(), has_ip)
         for a, b, nm in ((core, core_ref, "core"), (xo, xo_ref, "xattn")):
             err = (a.float().cpu() - b.float()).abs().max().item()
-            assert err <= 3e-2, f"step {(sp, dn, update, distill, extra)} {nm}: {err}"
+            assert err <= 2e-2, f"step {(sp, dn, update, distill, extra)} {nm}: {err}"
             assert _cosine(a, b) >= 0.9999, f"step {(sp, dn, update, distill, extra)} {nm}: cosine {_cosine(a, b)}"
         # what the cache holds afterwards must be what the reference's cache would hold
         if has_ip and (extra or sp > 0) and update:
             keep = S - L if distill else S
             got = ip.key_value_memory_dict[3][sp * L: sp * L + keep].float().cpu()
             want = cache_ref.mem[sp * L: sp * L + keep].float()
-            assert (got - want).abs().max() <= 3e-2
+            # (the two sides' projections come from different GEMM implementations, which may round a raw value to
+            # the other neighbour: within 2^-6 of the row's largest magnitude, K and V halves apart)
+            for half in (slice(0, D), slice(D, 2 * D)):
+                d = (got[..., half] - want[..., half]).abs()
+                assert torch.all(d <= want[..., half].abs().amax(dim=-1, keepdim=True) * 2.0 ** -6)
+
+
+def _cacheless_forward_vs_oracle(layer, dev, seed, tol=2e-2):
+    """One cache-less batch-1 forward of two chunks (one of them without text) against the oracle's layer."""
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+
+    hidden = layer.linear_qkv.q.weight.shape[1]
+    Hq, Hkv, D = layer.num_attention_heads, layer.num_query_groups_per_partition, 128
+    fr, H, W, dn = 2, 3, 4, 2
+    L = fr * H * W
+    S = dn * L
+    g = torch.Generator().manual_seed(seed)
+    hs = torch.randn(S, 1, hidden, generator=g).bfloat16()
+    lens = torch.tensor([7, 0])
+    mask = (torch.arange(8)[None] < lens[:, None]).float().view(dn, 1, 1, 8)
+    y = (torch.randn(int(lens.sum()), hidden, generator=g) * 0.5).bfloat16()
+    k_range, q_range = R.generate_kv_range_for_uncondition(dn, L), R.q_ranges_from_chunks(dn, L)
+    cross_p = P.build_cross_attn_params(mask.to(dev), L, 8)
+    meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=0, denoising_range_num=dn,
+                           range_num=dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=False,
+                           distill_nearly_clean_chunk=False, clip_token_nums=L, enable_cuda_graph=False,
+                           core_attn_params=P.build_core_attn_params(q_range.to(dev), k_range.to(dev), L),
+                           cross_attn_params=cross_p)
+    rope = LearnableRotaryEmbeddingCat(128, device=dev).get_embed_for_forward(dn * fr, H, W, 0, dn)
+    with torch.no_grad():
+        core, xo = layer(hs.to(dev), y.to(dev), None, rope, meta)
+    core_ref, xo_ref = _oracle_layer(layer, hs, y, O.rope_for_forward(dn * fr, H, W, 0, dn), 0, L, k_range.numpy(),
+                                     q_range.numpy(), O.KVCacheModel(S, Hkv, D), False, False, False,
+                                     cross_p.cu_seqlens_q.cpu(), cross_p.cu_seqlens_kv.cpu(), has_ip=False)
+    for a, b, nm in ((core, core_ref, "core"), (xo, xo_ref, "xattn")):
+        assert torch.isfinite(a).all(), nm
+        err = (a.float().cpu() - b.float()).abs().max().item()
+        assert err <= tol and _cosine(a, b) >= 0.9999, (nm, err, _cosine(a, b))
+
+
+def test_layer_follows_rewritten_norm_parameters_and_falls_back_above_the_bound(dev):
+    """The score bounds (a promise to kernels that keep no running maximum) and the constant e4m3 scales are derived
+    from the norm parameters and cached: after a parameter is rewritten, by copy_, by load_state_dict (in place and
+    with assign=True, the reference loader's form, inference/infra/checkpoint/checkpointing.py:168) or through .data
+    followed by invalidate_cached_parameters(), they must follow, and the forward must still match the oracle.
+    Gains that push a bound past MAGI_SCORE_BOUND_MAX make the layer fall back to the online-softmax kernel (and the
+    cross attention to its two-launch form); last_forward_kernels records the choice."""
+    import math
+
+    hidden, Hq, Hkv, D = 256, 6, 2, 128
+    layer = _make_layer(dev, hidden, Hq, Hkv, seed=21)
+    premul = D ** -0.5 * math.log2(math.e)
+
+    def expected(rotary_half=48):
+        b = lambda qn, kn, r: 1.01 * premul * MOD.qk_score_bound(qn, kn, r)
+        sc = (M.pow2_scale_for(premul * layer.q_layernorm.output_norm_bound()), M.pow2_scale_for(layer.k_layernorm.output_norm_bound()))
+        for ln in (layer.q_layernorm, layer.k_layernorm, layer.q_layernorm_xattn, layer.k_layernorm_xattn):
+            ln.invalidate_cached_parameters()  # (recomputed from the parameters as they are now)
+        return (b(layer.q_layernorm, layer.k_layernorm, rotary_half), b(layer.q_layernorm_xattn, layer.k_layernorm_xattn, 0)), sc
+
+    _cacheless_forward_vs_oracle(layer, dev, 1)
+    b0, s0 = layer.score_bounds(), layer.fp8_operand_scales()
+    assert max(b0) <= M.MAGI_SCORE_BOUND_MAX and "bounded" in layer.last_forward_kernels["core"]
+    assert "bounded" in layer.last_forward_kernels["cross"]
+    g = torch.Generator().manual_seed(5)
+    # 1. in-place copy_ under no_grad (advances the version counter)
+    with torch.no_grad():
+        layer.q_layernorm.weight.copy_(torch.randn(D, generator=g) * 0.4)
+    b1, s1 = layer.score_bounds(), layer.fp8_operand_scales()
+    assert b1[0] != b0[0] and b1[1] == b0[1]
+    _cacheless_forward_vs_oracle(layer, dev, 2)
+    want_b, want_s = expected()
+    assert b1 == pytest.approx(want_b) and s1 == want_s
+    # 2. a write through .data is invisible to the version counter: the caller invalidates
+    layer.k_layernorm.weight.data.copy_(torch.randn(D, generator=g) * 0.4)
+    layer.k_layernorm.bias.data.copy_(torch.randn(D, generator=g) * 0.5)
+    layer.invalidate_cached_parameters()
+    b2, s2 = layer.score_bounds(), layer.fp8_operand_scales()
+    want_b, want_s = expected()
+    assert b2 == pytest.approx(want_b) and s2 == want_s and b2[0] != b1[0]
+    _cacheless_forward_vs_oracle(layer, dev, 3)
+    # 3. load_state_dict in place, then with assign=True (new Parameter objects): large gains, bound above the limit
+    sd = {k_: v_.clone() for k_, v_ in layer.state_dict().items()}
+    sd["q_layernorm.weight"] = torch.full((D,), 1.6, device=dev)         # gamma + 1 = 2.6
+    sd["k_layernorm.weight"] = torch.full((D,), 1.5, device=dev)
+    layer.load_state_dict(sd)
+    b3 = layer.score_bounds()
+    assert b3[0] > M.MAGI_SCORE_BOUND_MAX and b3 == pytest.approx(expected()[0])
+    _cacheless_forward_vs_oracle(layer, dev, 4, tol=3e-2)  # (sharper softmax: outputs approach single V rows)
+    assert "online" in layer.last_forward_kernels["core"] and "bounded" in layer.last_forward_kernels["cross"]
+    sd = {k_: v_.clone() for k_, v_ in layer.state_dict().items()}
+    sd["q_layernorm.weight"] = torch.randn(D, generator=g).to(dev) * 0.1
+    sd["k_layernorm.weight"] = torch.randn(D, generator=g).to(dev) * 0.1
+    sd["q_layernorm_xattn.weight"] = torch.full((D,), 2.0, device=dev, dtype=torch.bfloat16)
+    sd["k_layernorm_xattn.weight"] = torch.full((D,), 2.0, device=dev, dtype=torch.bfloat16)
+    layer.load_state_dict(sd, assign=True)
+    b4 = layer.score_bounds()
+    assert b4[0] <= M.MAGI_SCORE_BOUND_MAX < b4[1] and b4 == pytest.approx(expected()[0])
+    assert layer.fp8_operand_scales() == expected()[1]
+    _cacheless_forward_vs_oracle(layer, dev, 5, tol=3e-2)
+    assert "bounded" in layer.last_forward_kernels["core"] and "online" in layer.last_forward_kernels["cross"]
 
 
 def test_layer_batched_cacheless_pass(dev):
@@ -506,8 +606,9 @@ def test_layer_with_fp8_self_attention_and_fp8_cache(dev, fast_exp2):
 def test_fp8_layer_prepares_its_operands_in_two_launches(dev):
     """Between the GEMM of the projections and the fp8 attention kernel the layer issues exactly two kernels: the prologue
     with e4m3 outputs (q, and k into the cache rows) and the one-launch V quantiser; no absmax / conversion
-    passes and no torch elementwise kernels.  Read from a kernel trace of one steady-state forward (skipped when
-    the profiler records no device activity)."""
+    passes and no torch elementwise kernels.  The library's own launch counter gives the number of its launches per
+    steady-state forward (six: input norm, prologue, V quantiser, fp8 attention, text-side k norm, cross attention);
+    a kernel trace of the same forward, when the profiler records device activity, names what lies between them."""
     from torch.profiler import ProfilerActivity, profile
     from magi_attn.rope import LearnableRotaryEmbeddingCat
 
@@ -540,14 +641,16 @@ def test_fp8_layer_prepares_its_operands_in_two_launches(dev):
     step(0, 3, True, True)
     torch.cuda.synchronize()
     for args in ((1, 3, True, True), (2, 3, True, False)):  # with and without rows that are not persisted
+        n0 = M.lib().magi_launch_count()
         with profile(activities=[ProfilerActivity.CUDA]) as prof:
             step(*args)
             torch.cuda.synchronize()
+        assert M.lib().magi_launch_count() - n0 == 6
         evs = sorted((e for e in prof.events() if e.device_type == torch.autograd.DeviceType.CUDA and "Memcpy" not in e.name
                       and "Memset" not in e.name), key=lambda e: e.time_range.start)
         names = [e.name for e in evs]
-        if not names:
-            pytest.skip("the profiler recorded no device activity")
+        if not names:  # (no device activity recorded: the launch count above is the check)
+            continue
         attn = [i for i, n in enumerate(names) if "attn_fwd_fp8_kernel" in n]
         assert len(attn) == 1, names
         ln = max(i for i, n in enumerate(names[:attn[0]]) if "layer_norm_kernel" in n)

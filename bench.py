@@ -485,8 +485,12 @@ def secondary_legs(inp, dev, steps):
     res["online_softmax_unscaled_q"] = entry(ms, core_fl, "attn_fwd_bf16_kernel (32 rows per wavefront, running maximum)")
     ms = timed(lambda: M.range_attention(q_unscaled, k, v, inp["q_ranges"], inp["k_ranges"], L, out=inp["out"],
                                          return_lse=False, score_bound=SCORE_BOUND), steps)
-    res["bounded_unscaled_q_scale_on_load"] = entry(ms, core_fl, "attn_fwd_bf16_w64_kernel (q scaled while loaded)")
+    res["bounded_unscaled_q_scale_on_load"] = entry(ms, core_fl, "attn_fwd_bf16_x16_kernel (q scaled while loaded)")
     del q_unscaled
+    # the bounded kernel's 32x32x16-MFMA form (MAGI_ATTN_BOUNDED_MFMA32) on the headline's inputs: same box, same run
+    ms = timed(lambda: M.range_attention(inp["q"], k, v, inp["q_ranges"], inp["k_ranges"], L, out=inp["out"],
+                                         return_lse=False, q_prescaled=True, score_bound=SCORE_BOUND, bounded_mfma32=True), steps)
+    res["bounded_mfma_32x32x16_form"] = entry(ms, core_fl, "attn_fwd_bf16_w64_kernel (64 rows per wavefront on v_mfma_f32_32x32x16)")
     # restore the headline's output (the accuracy legs compare inp["out"])
     M.range_attention(inp["q"], k, v, inp["q_ranges"], inp["k_ranges"], L, out=inp["out"], return_lse=False,
                       q_prescaled=True, score_bound=SCORE_BOUND)
@@ -497,7 +501,7 @@ def secondary_legs(inp, dev, steps):
         scratch = torch.empty_like(inp["out"])
         ms = timed(lambda: M.range_attention(inp["q"], k, v, inp["q_ranges"], krd, L, out=scratch, return_lse=False,
                                              q_prescaled=True, score_bound=SCORE_BOUND), steps)
-        res["sliding_window_noise2clean_5_4_3_2"] = entry(ms, fl, "attn_fwd_bf16_w64_kernel")
+        res["sliding_window_noise2clean_5_4_3_2"] = entry(ms, fl, "attn_fwd_bf16_x16_kernel")
         res["sliding_window_noise2clean_5_4_3_2"]["k_ranges"] = kr.numpy().tolist()
         del scratch
         small = build_inputs("480p-4.5B", dev)
@@ -510,7 +514,7 @@ def secondary_legs(inp, dev, steps):
             run_step(small, ev[s_])
         torch.cuda.synchronize()
         ms = float(np.mean([e["core"][0].elapsed_time(e["core"][1]) for e in ev]))
-        res["layer_480p_4.5B"] = entry(ms, fl, "attn_fwd_bf16_w64_kernel")
+        res["layer_480p_4.5B"] = entry(ms, fl, "attn_fwd_bf16_x16_kernel")
         res["layer_480p_4.5B"]["workload"] = (f"Q {small['S']} tok x {small['Hq']} heads over K/V "
                                               f"{(small['sp'] + small['dn']) * small['L']} tok x {small['Hkv']} heads")
     return res
@@ -592,7 +596,7 @@ def main():
                                f"+ T5 cross-attention (lens {inp['t5_lens'].tolist()})"
                                + ("" if args.kv_window == "default" else f", sliding-window key ranges {inp['k_ranges_host'].tolist()}"),
                    "core_flops": core_fl, "cross_flops": cross_fl},
-        "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_w64_kernel" if args.core_kernel == "bounded" else "attn_fwd_bf16_kernel", "achieved": round(core_tflops, 2),
+        "roofline": {"bound": "mfma", "kernel": "attn_fwd_bf16_x16_kernel" if args.core_kernel == "bounded" else "attn_fwd_bf16_kernel", "achieved": round(core_tflops, 2),
                      "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(core_tflops / PEAK_BF16_TFLOPS, 4),
                      "traffic": traffic.get("core") if args.kv_window == "default" else None,
                      "traffic_source": TRAFFIC_SOURCE, "ms": round(kern_ms["core"], 3),
@@ -609,7 +613,7 @@ def main():
                               "ms": round(kern_ms["prologue"], 4)},
         # the T5 cross attention launch (q norm inside the kernel): ~13 key tiles per query tile, so Q / O streaming
         # and the per-workgroup ramp weigh as much as the MFMAs; priced against both roofs
-        "roofline_cross": {"bound": "mfma", "kernel": "attn_fwd_bf16_w64_kernel (q_norm)", "achieved": round(cross_tflops, 2),
+        "roofline_cross": {"bound": "mfma", "kernel": "attn_fwd_bf16_x16_kernel (q_norm)", "achieved": round(cross_tflops, 2),
                            "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": round(cross_tflops / PEAK_BF16_TFLOPS, 4),
                            "hbm_gbs": round(cross_gbs, 1), "hbm_frac": round(cross_gbs / PEAK_HBM_GBS, 4),
                            "traffic": traffic.get("cross"), "traffic_source": TRAFFIC_SOURCE,

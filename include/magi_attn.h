@@ -49,6 +49,12 @@ extern "C" {
  * per-score multiply and, where it has an instantiation for it, lets the score MFMAs accumulate onto the negated
  * running maximum; softmax_scale is ignored.  No counterpart in the reference, whose kernels take unscaled q. */
 #define MAGI_ATTN_Q_PRESCALED 2
+/* bf16 with MAGI_ATTN_Q_PRESCALED and a score_bound in force: run the bounded-score kernel on v_mfma_f32_32x32x16
+ * instead of the default 16x16x32.  Same results up to the order of fp32 additions.  The default shape spends less
+ * energy per FLOP, which is what counts on a part at its board power limit (+3 % on the 720p layer, 0 to +6 % from box
+ * to box); the 32x32x16 form issues half as many MFMAs and is the better one where the clock, not the power, is
+ * capped.  512-row workgroups (q_tile_rows) always use it. */
+#define MAGI_ATTN_BOUNDED_MFMA32 8
 
 #define MAGI_RANGES_PAIRS 0 /* int32 [n, 2]: range i = [r[2i], r[2i+1])          */
 #define MAGI_RANGES_CU 1    /* int32 [n + 1] cumulative: range i = [r[i], r[i+1]) */

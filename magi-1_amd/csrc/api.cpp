@@ -168,10 +168,11 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   a.n_ranges = p->n_ranges;
   a.ranges_mode = p->ranges_mode;
   // Kernel choice for bf16.
-  //  * Scores with a promised bound (score_bound): the kernel without a running maximum that holds 64 query rows per
-  //    wavefront (every K / V fragment read from LDS feeds two MFMAs); 256-row workgroups (4 waves, two per CU:
-  //    the two waves of a SIMD belong to different workgroups and drift out of step, so one computes scores while
-  //    the other is in its softmax).
+  //  * Scores with a promised bound (score_bound): the kernels without a running maximum that hold 64 query rows per
+  //    wavefront; 256-row workgroups (4 waves, two per CU: the two waves of a SIMD belong to different workgroups
+  //    and drift out of step, so one computes scores while the other is in its softmax) on v_mfma_f32_16x16x32
+  //    (the part is power limited and that shape takes less energy per FLOP; measured +3 % on the 720p layer,
+  //    between 0 and +6 % from box to box); the 32x32x16 form on request and for 512-row workgroups.
   //  * Otherwise 32 rows per wavefront with the online softmax: 384-row workgroups (12 waves, one workgroup per CU,
   //    every K / V tile fetched once for three times as many rows and one barrier per tile) pay on grids of many
   //    rounds with long key ranges (measured: +3 % at 43 rounds, +1 % at 9.4, -3 % at 5.3); small grids and short
@@ -183,6 +184,9 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   // a bound stated for unscaled q (what the reference's callers pass): the kernel applies the softmax scale while it
   // loads q, after which the scores are exp2 exponents as with MAGI_ATTN_Q_PRESCALED
   const bool scale_q = bounded && !q_norm && !(p->flags & MAGI_ATTN_Q_PRESCALED);
+  const bool mfma32 = (p->flags & MAGI_ATTN_BOUNDED_MFMA32) != 0;
+  if (mfma32 && !(bounded && (p->flags & MAGI_ATTN_Q_PRESCALED)))
+    return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_BOUNDED_MFMA32 goes with bf16, MAGI_ATTN_Q_PRESCALED and a score_bound in force");
   if (p->dtype == MAGI_DTYPE_BF16) {
     const double wg384 = (double)p->Hq * p->n_ranges * ((p->max_seqlen_q + 383) / 384);
     const bool long_keys = p->max_seqlen_k == 0 || p->max_seqlen_k >= 4096;  // (0 = not stated)
@@ -224,6 +228,8 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   hipError_t e;
   if (p->dtype != MAGI_DTYPE_BF16)
     e = magi::launch_attn_fwd_fp8(a, static_cast<hipStream_t>(stream));
+  else if (bounded && a.block_m == 256 && !mfma32)
+    e = magi::launch_attn_fwd_bf16_x16(a, static_cast<hipStream_t>(stream));
   else if (bounded)
     e = magi::launch_attn_fwd_bf16_w64(a, static_cast<hipStream_t>(stream));
   else

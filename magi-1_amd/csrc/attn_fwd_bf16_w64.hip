@@ -14,6 +14,10 @@
 // fragments that alternates between K and V^T fragments in the order the MFMAs consume them; the first V^T
 // fragments of a half are on their way while its softmax runs.
 //
+// The library's default bounded-score kernel is the 16x16x32 form of attn_fwd_bf16_x16.hip (less energy per FLOP on
+// this power-limited part); this 32x32x16 form issues half as many MFMAs and serves the 512-row workgroups and
+// callers that ask for it (MAGI_ATTN_BOUNDED_MFMA32).  q must carry the softmax scale (MAGI_ATTN_Q_PRESCALED).
+//
 // Every instantiation is for BOUNDED scores (magi_attn_args.score_bound): the caller guarantees
 // |q . k| <= score_bound (an exp2 exponent, q carrying softmax_scale * log2(e) by the time the MFMAs see it),
 // small enough that 2^score neither overflows nor underflows in fp32 / bf16.  The softmax is shift invariant, so
@@ -52,12 +56,7 @@ __device__ __forceinline__ float keep_lanes(float p, unsigned long long m) {
   return r;
 }
 
-// QMODE: what q holds.  0: q as the score MFMAs take it (pre-scaled by the caller, or BOUNDED is off and the scale is
-// applied per score).  1: the raw query projection: per-(token, head) norm in fp32 while it is loaded, times the
-// softmax scale, one rounding to bf16.  2: unscaled bf16 q as the reference's callers pass it: multiplied by the
-// softmax scale while it is loaded (a second rounding to bf16: 2^-9 relative per element, the size of the first).
-constexpr int Q_AS_IS = 0, Q_NORM = 1, Q_SCALE = 2;
-template <int NW, int OCC, int VPRE, int RD, int QMODE = Q_AS_IS>
+template <int NW, int OCC, int VPRE, int RD>
 __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const AttnKernArgs a) {
   constexpr int BM = 64 * NW;
   constexpr int LW = 4;                 // waves that load tiles (the last LW of the workgroup)
@@ -95,65 +94,6 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const A
 #pragma unroll
     for (int kk = 0; kk < 8; ++kk) qf[b][kk] = *(const bf16x8*)(qp + kk * 32);
   }
-  if constexpr (QMODE == Q_SCALE) {
-    const float cs = a.scale_log2;
-#pragma unroll
-    for (int b = 0; b < 2; ++b)
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) qf[b][kk][e] = (__bf16)((float)qf[b][kk][e] * cs);
-  }
-  if constexpr (QMODE == Q_NORM) {
-    // q holds the raw projection: per-(token, head) norm over the 128 features in fp32, times the softmax scale,
-    // one rounding to bf16 (the cross-attention query norm, folded into this kernel's Q load).  A row's features
-    // are spread over the lane pair (i, 0), (i, 1): 64 each, feature 16 kk + 8 g + e in fragment kk, element e.
-    const float inv_d = 1.f / 128.f;
-    float mean[2], rstd[2];
-#pragma unroll
-    for (int b = 0; b < 2; ++b) {
-      float sum = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) sum += (float)qf[b][kk][e];
-      sum += __shfl_xor(sum, 32);
-      mean[b] = a.q_norm_kind == 0 ? sum * inv_d : 0.f;  // (RMS form: no centring)
-      float sq = 0.f;
-#pragma unroll
-      for (int kk = 0; kk < 8; ++kk)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float d = (float)qf[b][kk][e] - mean[b];
-          sq += d * d;
-        }
-      sq += __shfl_xor(sq, 32);
-      rstd[b] = __builtin_amdgcn_rsqf(sq * inv_d + a.q_norm_eps) * a.scale_log2;
-    }
-    // (one fragment index at a time, so that the parameters of one fragment are all that is in registers)
-#pragma unroll
-    for (int kk = 0; kk < 8; ++kk) {
-      __builtin_amdgcn_sched_barrier(0);
-      const f32x4* gp = (const f32x4*)(a.q_norm_gamma + 16 * kk + 8 * g);
-      const f32x4 g0 = gp[0], g1 = gp[1];
-      f32x4 b0 = {0.f, 0.f, 0.f, 0.f}, b1 = b0;
-      if (a.q_norm_beta) {
-        const f32x4* bp = (const f32x4*)(a.q_norm_beta + 16 * kk + 8 * g);
-        b0 = bp[0];
-        b1 = bp[1];
-      }
-#pragma unroll
-      for (int b = 0; b < 2; ++b)
-#pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          const float gm = (e < 4 ? g0[e & 3] : g1[e & 3]) + 1.f;
-          const float bt = (e < 4 ? b0[e & 3] : b1[e & 3]) * a.scale_log2;
-          qf[b][kk][e] = (__bf16)(((float)qf[b][kk][e] - mean[b]) * rstd[b] * gm + bt);
-        }
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  }
-
   // ---- K/V tile loader: loading wave wl fills rows 4*(wl + LW*j) .. +3; lane l sits at row +(l >> 4), slot l & 15 ----
   const int wl = w - (NW - LW);
   const long ks_t = a.ks_t, vs_t = a.vs_t;
@@ -388,11 +328,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const A
 
 hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream) {
   const dim3 grid(a.per_xcd * 8u);
-  if (a.q_norm_gamma)  // raw q, normalised while it is loaded (cross attention)
-    hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 2, 0, 4, Q_NORM>), grid, dim3(256), 0, stream, a);
-  else if (a.flags & ATTN_SCALE_Q)  // unscaled q, scaled while it is loaded (the reference-shaped callables)
-    hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 2, 0, 4, Q_SCALE>), grid, dim3(256), 0, stream, a);
-  else if (a.block_m == 512)  // 8 waves, one workgroup per CU: every K / V tile fetched once for 512 rows
+  if (a.block_m == 512)  // 8 waves, one workgroup per CU: every K / V tile fetched once for 512 rows
     hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<8, 1, 0, 4>), grid, dim3(512), 0, stream, a);
   else  // 4 waves, two workgroups per CU
     hipLaunchKernelGGL((attn_fwd_bf16_w64_kernel<4, 2, 0, 4>), grid, dim3(256), 0, stream, a);

@@ -48,6 +48,7 @@ constexpr int ATTN_SCALE_Q = 1 << 9;
 
 hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream);
 hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream);
+hipError_t launch_attn_fwd_bf16_x16(const AttnKernArgs& a, hipStream_t stream);
 hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream);
 
 struct PrologueKernArgs {

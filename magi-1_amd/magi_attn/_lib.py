@@ -21,6 +21,7 @@ MAGI_NORM_NONE = 2
 MAGI_ATTN_FP8_POW2_PRESCALED = 1
 MAGI_ATTN_Q_PRESCALED = 2
 MAGI_ATTN_FP8_FAST_EXP2 = 4
+MAGI_ATTN_BOUNDED_MFMA32 = 8
 MAGI_SCORE_BOUND_MAX = 64.0
 
 

@@ -73,6 +73,7 @@ def range_attention(
     q_prescaled: bool = False,
     score_bound: float = 0.0,
     q_tile_rows: int = 0,
+    bounded_mfma32: bool = False,
     q_norm: Optional[tuple] = None,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = True,
@@ -95,6 +96,7 @@ def range_attention(
     factor is already in q); see magi_attn_args.score_bound.  Without q_prescaled the kernel applies the scale while
     it loads q.
     q_tile_rows: force a workgroup shape (0 = the library's choice); see magi_attn_args.q_tile_rows.
+    bounded_mfma32 (with q_prescaled and score_bound): the 32x32x16 form of the bounded kernel, MAGI_ATTN_BOUNDED_MFMA32.
     q_norm: (gamma, beta or None, eps[, norm_kind]): q is the raw projection, normalised per (token, head) row inside
     the kernel (fp32, zero-centred gamma) and scaled by softmax_scale * log2(e); needs score_bound.
     """
@@ -171,7 +173,7 @@ def range_attention(
     a.scale_chunk_tokens = int(scale_chunk_tokens)
     a.softmax_scale = 0.0 if softmax_scale is None else float(softmax_scale)
     a.flags = ((L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0) | (L.MAGI_ATTN_Q_PRESCALED if q_prescaled else 0)
-               | (L.MAGI_ATTN_FP8_FAST_EXP2 if fp8_fast_exp2 else 0))
+               | (L.MAGI_ATTN_FP8_FAST_EXP2 if fp8_fast_exp2 else 0) | (L.MAGI_ATTN_BOUNDED_MFMA32 if bounded_mfma32 else 0))
     a.score_bound = float(score_bound)
     a.q_tile_rows = int(q_tile_rows)
     keep = None

@@ -57,11 +57,14 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("rows", [0, 256, 512])
+@pytest.mark.parametrize("rows", [0, 256, 512, "mfma32"])
 @pytest.mark.parametrize("L,dn,sp,Hq,Hkv", CASES)
 def test_bounded_chunk_causal_parity(dev, L, dn, sp, Hq, Hkv, rows):
-    """rows: the workgroup shape (magi_attn_args.q_tile_rows; 0 = the library's choice, which is 256 rows on inputs
-    this small): 256 = 4 waves, 512 = 8 waves of 64 query rows."""
+    """rows: the workgroup shape (magi_attn_args.q_tile_rows; 0 = the library's choice, 256 rows): 256 = 4 waves of 64
+    query rows on the 16x16x32 MFMA, 512 = 8 waves on the 32x32x16 MFMA; "mfma32" = 4 waves on the 32x32x16 MFMA
+    (MAGI_ATTN_BOUNDED_MFMA32)."""
+    mfma32 = rows == "mfma32"
+    rows = 0 if mfma32 else rows
     q, k, v, bound = _inputs(dn * L, (sp + dn) * L, Hq, Hkv, seed=4321 + L)
     assert bound <= M.MAGI_SCORE_BOUND_MAX
     qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
@@ -69,7 +72,7 @@ def test_bounded_chunk_causal_parity(dev, L, dn, sp, Hq, Hkv, rows):
     lse_ref = O.range_attention_lse(q, k, v, qr, kr, softmax_scale=LN2)
     tq, tk = _ranges(dev, qr, kr)
     out, lse = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, int(kr.max() - kr.min()),
-                                 q_prescaled=True, score_bound=bound, q_tile_rows=rows)
+                                 q_prescaled=True, score_bound=bound, q_tile_rows=rows, bounded_mfma32=mfma32)
     _cmp(out, ref, f"L={L}")
     assert (lse.cpu() - lse_ref).abs().max() < 5e-3
     # against the online-softmax kernel on the same inputs: the same softmax up to the rounding of p to bf16
@@ -117,14 +120,15 @@ def test_bounded_varlen_segments_with_empty_and_ragged_keys(dev):
     _cmp(out, ref)
 
 
-def test_bounded_cache_views_two_segments_and_grouped_output(dev):
+@pytest.mark.parametrize("mfma32", [False, True])
+def test_bounded_cache_views_two_segments_and_grouped_output(dev, mfma32):
     """K / V read in place from an interleaved cache, the key axis split into [cache prefix | side buffer] at
     tile-unfriendly places, and the output written in the two-level head layout: all bit-identical to the plain call."""
     L, sp, dn, Hq, Hkv, D = 90, 2, 3, 8, 2, 128
     q, k, v, bound = _inputs(dn * L, (sp + dn) * L, Hq, Hkv, seed=8)
     qr, kr = O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L)
     tq, tk = _ranges(dev, qr, kr)
-    kw = dict(q_prescaled=True, score_bound=bound)
+    kw = dict(q_prescaled=True, score_bound=bound, bounded_mfma32=mfma32)
     base = M.range_attention(q.to(dev), k.to(dev), v.to(dev), tq, tk, L, **kw)[0]
     _cmp(base, O.range_attention(q, k, v, qr, kr, softmax_scale=LN2))
     cache = torch.cat([k, v], -1).to(dev)
@@ -157,6 +161,10 @@ def test_score_bound_argument_checks(dev):
         M.range_attention(q, q, q, r, r, 4, q_prescaled=True, score_bound=8.0, q_tile_rows=384)
     with pytest.raises(M.MagiError):
         M.range_attention(q, q, q, r, r, 4, q_tile_rows=512)
+    with pytest.raises(M.MagiError):  # the 32x32x16 form takes pre-scaled q and a bound
+        M.range_attention(q, q, q, r, r, 4, score_bound=8.0, bounded_mfma32=True)
+    with pytest.raises(M.MagiError):
+        M.range_attention(q, q, q, r, r, 4, q_prescaled=True, bounded_mfma32=True)
 
 
 @pytest.mark.parametrize("L,dn,sp,Hq,Hkv", CASES)

@@ -1,10 +1,11 @@
 """Benchmark-size parity of the kernels the layer and the benchmark actually launch.
 
 Every shipped bf16 instantiation runs the 480p and the 720p layer shapes and the ragged four-video batch: the
-online-softmax kernel (32 rows per wavefront; what a caller without a score bound gets), the bounded-score kernel
-(64 rows per wavefront, no running maximum; what FullyParallelAttention.forward and bench.py launch) in its 256- and
-512-row workgroup shapes, and the bounded kernel with the softmax scale applied while q is loaded (what the four
-reference-shaped callables select when given score_bound=).  The fused prologue runs at S = 86400 x 56 head rows into
+online-softmax kernel (32 rows per wavefront; what a caller without a score bound gets), the bounded-score kernels
+(64 rows per wavefront, no running maximum): the 16x16x32-MFMA form with 256-row workgroups that
+FullyParallelAttention.forward and bench.py launch, the 32x32x16-MFMA form with 256- and 512-row workgroups, and the
+default form with the softmax scale applied while q is loaded (what the four reference-shaped callables select when
+given score_bound=).  The fused prologue runs at S = 86400 x 56 head rows into
 a 259200-row cache, and one FullyParallelAttention.forward runs at hidden 6144 / 48 / 8 heads over a resident arena.
 
 Outputs of this size are checked on row subsamples.  Query rows are independent of each other, so fp32 attention of
@@ -45,6 +46,7 @@ VARIANTS = {
     "online-prescaled": (True, dict(q_prescaled=True)),
     "bounded-256": (True, dict(q_prescaled=True, score_bound=UNIT_GAIN_BOUND, q_tile_rows=0)),
     "bounded-512": (True, dict(q_prescaled=True, score_bound=UNIT_GAIN_BOUND, q_tile_rows=512)),
+    "bounded-mfma32": (True, dict(q_prescaled=True, score_bound=UNIT_GAIN_BOUND, bounded_mfma32=True)),
     "bounded-scale-on-load": (False, dict(score_bound=UNIT_GAIN_BOUND)),
 }
 
@@ -149,7 +151,7 @@ def test_core_attention_full_size(layer_case, variant):
     assert (o1.float() - 1).abs().max().item() <= 2 ** -7
 
 
-@pytest.mark.parametrize("variant", ["online", "bounded-256", "bounded-512", "bounded-scale-on-load"])
+@pytest.mark.parametrize("variant", ["online", "bounded-256", "bounded-512", "bounded-mfma32", "bounded-scale-on-load"])
 def test_full_size_ragged_batch_with_cross_attention(dev, variant):
     """Four videos packed on one token axis with 1, 2, 3 and 4 active 9360-token chunks and 0-6 cached prefix chunks
     each (seeded), chunk-causal inside each video (24 / 8 heads), then cross attention from every video token to that

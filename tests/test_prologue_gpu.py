@@ -335,8 +335,10 @@ def _cacheless_forward_vs_oracle(layer, dev, seed, tol=2e-2):
                                      cross_p.cu_seqlens_q.cpu(), cross_p.cu_seqlens_kv.cpu(), has_ip=False)
     for a, b, nm in ((core, core_ref, "core"), (xo, xo_ref, "xattn")):
         assert torch.isfinite(a).all(), nm
-        err = (a.float().cpu() - b.float()).abs().max().item()
-        assert err <= tol and _cosine(a, b) >= 0.9999, (nm, err, _cosine(a, b))
+        d = (a.float().cpu() - b.float()).abs()
+        # (max-abs bar, or one bf16 ulp of the value where that is larger: outputs of magnitude 4 and more)
+        assert torch.all(d <= torch.clamp(b.float().abs() * 2.0 ** -7, min=tol)), (nm, d.max().item())
+        assert _cosine(a, b) >= 0.9999, (nm, _cosine(a, b))
 
 
 def test_layer_follows_rewritten_norm_parameters_and_falls_back_above_the_bound(dev):
@@ -388,8 +390,9 @@ def test_layer_follows_rewritten_norm_parameters_and_falls_back_above_the_bound(
     b3 = layer.score_bounds()
     assert b3[0] > M.MAGI_SCORE_BOUND_MAX and b3 == pytest.approx(expected()[0])
     # (the scores are four times as large, and with them the effect of q's and k's rounding to bf16, which the layer
-    # and the oracle do at different points: q after / before the softmax scale)
-    _cacheless_forward_vs_oracle(layer, dev, 4, tol=3e-2)
+    # and the oracle do at different points: q after / before the softmax scale; the softmax is sharp, so outputs
+    # are close to single V rows of magnitude 2-4, where two bf16 ulps are 0.031)
+    _cacheless_forward_vs_oracle(layer, dev, 4, tol=4e-2)
     assert "online" in layer.last_forward_kernels["core"] and "bounded" in layer.last_forward_kernels["cross"]
     sd = {k_: v_.clone() for k_, v_ in layer.state_dict().items()}
     sd["q_layernorm.weight"] = torch.randn(D, generator=g).to(dev) * 0.1
@@ -400,7 +403,7 @@ def test_layer_follows_rewritten_norm_parameters_and_falls_back_above_the_bound(
     b4 = layer.score_bounds()
     assert b4[0] <= M.MAGI_SCORE_BOUND_MAX < b4[1] and b4 == pytest.approx(expected()[0])
     assert layer.fp8_operand_scales() == expected()[1]
-    _cacheless_forward_vs_oracle(layer, dev, 5, tol=3e-2)
+    _cacheless_forward_vs_oracle(layer, dev, 5, tol=4e-2)
     assert "bounded" in layer.last_forward_kernels["core"] and "online" in layer.last_forward_kernels["cross"]
 
 

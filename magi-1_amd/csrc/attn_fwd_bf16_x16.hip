@@ -51,13 +51,6 @@ __device__ __forceinline__ int swz(int base, int tie) {
   return r;
 }
 
-// p in the lanes whose bit is set in the (wave-uniform) mask m, 0 elsewhere
-__device__ __forceinline__ float keep_lanes(float p, unsigned long long m) {
-  float r;
-  asm("v_cndmask_b32 %0, 0, %1, %2" : "=v"(r) : "v"(p), "s"(m));
-  return r;
-}
-
 // QMODE: what q holds.  0: q as the score MFMAs take it (pre-scaled by the caller).  1: the raw query projection:
 // per-(token, head) norm in fp32 while it is loaded, times the softmax scale, one rounding to bf16.  2: unscaled
 // bf16 q as the reference's callers pass it: multiplied by the softmax scale while it is loaded (a second rounding
@@ -68,7 +61,7 @@ template <int QMODE>
 __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKernArgs a) {
   constexpr int NW = 4, BM = 64 * NW;
   constexpr int LOADS = BN / (4 * NW);  // direct loads per wave per matrix per tile (4 rows each)
-  constexpr int RD = 4;                 // operand fragments in flight between LDS and the MFMAs
+  constexpr int RING = 4;               // operand fragments in flight between LDS and the MFMAs
   // K and V double buffered in four separate LDS objects that are only named statically (an operand read then
   // never waits for the direct loads in flight to the other pair of slots)
   __shared__ __attribute__((aligned(1024))) unsigned char sK0[TILE_BYTES];
@@ -228,11 +221,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   const int r4 = n >> 2, c4 = n & 3;
   const int base_v = (4 * g + r4) * ROW_BYTES + ((((c4 >> 1) ^ ((4 * (g & 1) + r4) << 1))) << 4) + ((c4 & 1) << 3);
 
-  f32x4v o_acc[8][4];  // [d block][query block]
-#pragma unroll
-  for (int db = 0; db < 8; ++db)
-#pragma unroll
-    for (int qb = 0; qb < 4; ++qb) o_acc[db][qb] = f32x4v{0.f, 0.f, 0.f, 0.f};
+  f32x4v o_acc[8][4];  // [d block][query block]; zeroed below, right ahead of the first tile
   float l_run[4] = {0.f, 0.f, 0.f, 0.f};  // this lane's share of the row sums, per query block
   const bool wave_on = row0 < qe;
   const f32x4v zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -258,6 +247,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
         return __builtin_bit_cast(bf16x8, va);
       }
     };
+    constexpr int RD = RING;
     bf16x8 ring[RD];
     static_for<0, RD>([&](auto oc) __attribute__((always_inline)) { ring[decltype(oc)::value] = read_op(oc); });
     __builtin_amdgcn_sched_barrier(0);
@@ -267,31 +257,15 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
     static_for<0, 32>([&](auto oc) __attribute__((always_inline)) {
       constexpr int o = decltype(oc)::value;
       constexpr int t = o >> 4, j = o & 15;
-      // ---- softmax of half t (32 keys x 64 queries: 32 values per lane, one query per lane and query block) ----
-      // Keys past the end of the range hold copies of the last valid row (the loader clamps), so their scores are
-      // finite; their probabilities are set to zero after the exp.  One (key block, query block) piece at a time:
-      // four exponentials, their sum, two packed pairs of the P operand.
+      // ---- softmax of half t (32 keys x 64 queries: 32 values per lane, one query per lane and query block), one
+      // (key block, query block) piece at a time: four exponentials, their sum, two packed pairs of the P operand.
+      // (Keys past the end of the range need nothing here: their scores start from a large negative value, see below.)
       auto soft = [&](auto kc, auto qc) __attribute__((always_inline)) {
         constexpr int kb = decltype(kc)::value, qb = decltype(qc)::value;
-        const int left = ke - (k0 + 32 * t);  // valid keys in this half (may be <= 0)
-        auto prob = [&](float x, auto rc) __attribute__((always_inline)) -> float {
-          const float p = __builtin_amdgcn_exp2f(x);
-          if constexpr (decltype(ragged)::value) {
-            // register (kb, r) of the lanes of group g holds key 16 kb + 4 g + r of the half: which of the four
-            // 16-lane groups keep their value is a scalar question per register
-            constexpr int c0 = 16 * kb + decltype(rc)::value;
-            const unsigned long long m = (c0 < left ? 0x000000000000ffffull : 0ull) | (c0 + 4 < left ? 0x00000000ffff0000ull : 0ull) |
-                                         (c0 + 8 < left ? 0x0000ffff00000000ull : 0ull) | (c0 + 12 < left ? 0xffff000000000000ull : 0ull);
-            return keep_lanes(p, m);
-          }
-          return p;
-        };
         // Row sums in fp32 by plain additions on the unrounded values (rounding to bf16 is unbiased, so this is as
         // good a denominator; dot instructions would hold the matrix pipe up)
-        const float p0 = prob(sc[kb][qb][0], std::integral_constant<int, 0>{});
-        const float p1 = prob(sc[kb][qb][1], std::integral_constant<int, 1>{});
-        const float p2 = prob(sc[kb][qb][2], std::integral_constant<int, 2>{});
-        const float p3 = prob(sc[kb][qb][3], std::integral_constant<int, 3>{});
+        const float p0 = __builtin_amdgcn_exp2f(sc[kb][qb][0]), p1 = __builtin_amdgcn_exp2f(sc[kb][qb][1]);
+        const float p2 = __builtin_amdgcn_exp2f(sc[kb][qb][2]), p3 = __builtin_amdgcn_exp2f(sc[kb][qb][3]);
         l_run[qb] += (p0 + p1) + (p2 + p3);
         pf[qb][2 * kb] = pack_bf16x2(p0, p1);
         pf[qb][2 * kb + 1] = pack_bf16x2(p2, p3);
@@ -311,9 +285,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
       if constexpr (j < 8) {
         // scores: S^T[key][q] += K[key][32 kk ..] Q[q][32 kk ..]
         constexpr int kb = j >> 2, kk = j & 3;
+        // The accumulators of a key block start from 0.  In the ragged copy of the body, keys past the end of the
+        // range (whose LDS rows hold copies of the last valid key: the loader clamps) start from -1e4 instead: their
+        // scores stay far below any real one (|score| <= 64), 2^score is exactly 0, and neither the row sums nor
+        // the P operand see them.  Register r of the lanes of group g is key 16 kb + 4 g + r of the half.
+        f32x4v c0 = zero4;
+        if constexpr (decltype(ragged)::value && kk == 0) {
+          const int left = ke - (k0 + 32 * t) - 16 * kb - 4 * (l >> 4);  // valid keys from this lane's first one on
+#pragma unroll
+          for (int r = 0; r < 4; ++r) c0[r] = r < left ? 0.f : -1.0e4f;
+        }
 #pragma unroll
         for (int qb = 0; qb < 4; ++qb)
-          sc[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[o % RD], qf[qb][kk], kk == 0 ? zero4 : sc[kb][qb], 0, 0, 0);
+          sc[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[o % RD], qf[qb][kk], kk == 0 ? c0 : sc[kb][qb], 0, 0, 0);
       } else {
         // O^T[d][q] += V^T[d][key] P^T[key][q]
         constexpr int db = j - 8;
@@ -340,6 +324,21 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   const std::integral_constant<int, 1> slot1;
   issue_mat(ks + last * BN, sK0, false);
   issue_mat(ks + last * BN, sV0, true);
+  // The accumulators start from zeros the compiler cannot see through: left to fold them into the first tile's
+  // MFMAs it allocates that tile's registers differently from the steady-state body and spills two accumulators
+  // there, a round trip to scratch memory for every workgroup.  (Here, behind the tile requests, so that the 128
+  // registers are not held while q is loaded and normalised: the statement below pins the finished q fragments
+  // ahead of them, or the compiler sinks the norm arithmetic to its first use, behind the zeros.)
+  asm volatile("" ::"v"(qf[0][0]), "v"(qf[0][1]), "v"(qf[0][2]), "v"(qf[0][3]), "v"(qf[1][0]), "v"(qf[1][1]), "v"(qf[1][2]),
+               "v"(qf[1][3]), "v"(qf[2][0]), "v"(qf[2][1]), "v"(qf[2][2]), "v"(qf[2][3]), "v"(qf[3][0]), "v"(qf[3][1]),
+               "v"(qf[3][2]), "v"(qf[3][3]));
+#pragma unroll
+  for (int db = 0; db < 8; ++db)
+#pragma unroll
+    for (int qb = 0; qb < 4; ++qb) {
+      o_acc[db][qb] = f32x4v{0.f, 0.f, 0.f, 0.f};
+      asm volatile("" : "+v"(o_acc[db][qb]));
+    }
   // one tile: wait for it, request the next one (tile `nxt` of the range, if any) into the other slot pair, compute
   auto step = [&](int cur, int nxt, auto sc_, auto ragged) __attribute__((always_inline)) {
     constexpr int B = decltype(sc_)::value;

@@ -292,11 +292,10 @@ def test_attention_kernels_keep_their_registers():
     flags = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + csrc,
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wno-unused-command-line-argument",
              "--cuda-device-only", "-Rpass-analysis=kernel-resource-usage", "-c", "-o", os.devnull]
-    # The bf16 main loops must not spill.  The 16x16x32 kernel parks a few values around its ragged first tile and
-    # its q-norm / q-scale prologues (outside the steady-state loop): at most 64 bytes per lane, and none of the
-    # scratch instructions may sit inside a loop of the generated code (checked on the assembly below).
+    # The bf16 kernels must not spill at all (the 16x16x32 kernel once parked two accumulators around its first tile:
+    # outside the steady-state loop, but a round trip to scratch memory for every workgroup, 12 % more bytes written).
     for src, limit in (("attn_fwd_bf16.hip", 0), ("attn_fwd_fp8.hip", 24), ("attn_fwd_bf16_w64.hip", 0),
-                       ("attn_fwd_bf16_x16.hip", 64)):
+                       ("attn_fwd_bf16_x16.hip", 0)):
         r = subprocess.run([hipcc] + flags + [os.path.join(csrc, src)], capture_output=True, text=True, timeout=600)
         assert r.returncode == 0, r.stderr[-2000:]
         names = re.findall(r"Function Name: (\S+)", r.stderr)
@@ -310,20 +309,3 @@ def test_attention_kernels_keep_their_registers():
                 assert sc <= limit, f"{n}: {sc} bytes of scratch per lane"
                 assert vg <= 256
         assert seen >= 2
-    # the 16x16x32 kernel's spills lie outside its tile loops: in the assembly, no scratch access between a loop
-    # header label and the backward branch that closes it
-    asm = subprocess.run([hipcc] + [f for f in flags if not f.startswith("-Rpass") and f not in ("-c",)][:-2] +
-                         ["-S", "-o", "-", os.path.join(csrc, "attn_fwd_bf16_x16.hip")], capture_output=True, text=True, timeout=600)
-    assert asm.returncode == 0, asm.stderr[-2000:]
-    # (the compiler annotates every basic-block label that belongs to a loop: "Loop Header", "in Loop", "Parent Loop")
-    in_loop, loop_blocks, n_scratch = False, 0, 0
-    for ln in asm.stdout.splitlines():
-        if re.match(r"^\.LBB\d+_\d+:", ln):
-            in_loop = "Loop" in ln
-            loop_blocks += in_loop
-        elif re.match(r"^\S+:", ln):  # a function label
-            in_loop = False
-        elif "scratch_" in ln:
-            n_scratch += 1
-            assert not in_loop, f"scratch access inside a loop: {ln.strip()}"
-    assert loop_blocks > 0, "no loop annotations found in the assembly"

@@ -87,9 +87,12 @@ class ClockSampler:
         if self._thread is not None:
             self._thread.join()
 
-    def result(self):
-        clk = [c for c, _ in self.samples if c]
-        pw = [p for _, p in self.samples if p]
+    def result(self, last_fraction=1.0):
+        """Medians over the samples (last_fraction < 1: over the last part of them only; the driver's metrics lag the
+        load by a few hundred milliseconds)."""
+        keep = self.samples[int(len(self.samples) * (1.0 - last_fraction)):]
+        clk = [c for c, _ in keep if c]
+        pw = [p for _, p in keep if p]
         return (float(np.median(clk)) if clk else None, float(np.median(pw)) if pw else None, len(self.samples))
 
 WORKLOADS = {
@@ -385,9 +388,26 @@ def projection_leg(inp, steps):
         M.qkv_proj_prologue(x, w, inp["rope"], z, z, z, z, Hq=Hq, Hkv=Hkv, Hqx=Hq, kv_out=kv_dst, n_cache_rows=S,
                             q_out=q_dst, qx_out=inp["xout"], q_premul=Q_PREMUL)
 
+    # the reference's fp8_quant layers: per linear (q, k, v, qx) its own input quantiser (div_clamp_to, one pass over x)
+    # and the library's fp8 GEMM, then the prologue on the four results
+    from magi_attn.module import PerTensorQuantizedFp8Linear
+    lins = []
+    row = 0
+    for n_out in (nq, nk, nk, nq):
+        lin = torch.nn.Linear(hidden, n_out, bias=False, dtype=torch.bfloat16, device=dev)
+        lin.weight.data = w[row:row + n_out]
+        lins.append(PerTensorQuantizedFp8Linear.from_linear(lin, 6.0))
+        row += n_out
+
+    def fp8_linears():
+        qr_, kr_, vr_, _ = (l_(x) for l_ in lins)
+        M.qk_prologue(qr_, kr_, vr_, inp["rope"], z, z, z, z, Hq=Hq, Hkv=Hkv, kv_out=kv_dst, n_cache_rows=S, q_out=q_dst,
+                      q_premul=Q_PREMUL)
+
     res = {"flop": flop, "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS}
     for name, fn in (("library_gemm", lambda: torch.mm(x, w.t(), out=raw)), ("library_gemm_then_prologue", two_step),
-                     ("gemm_with_prologue_epilogue", one_launch)):
+                     ("gemm_with_prologue_epilogue", one_launch),
+                     ("fp8_quant_linears_then_prologue", fp8_linears)):
         fn()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -419,7 +439,8 @@ def timed(fn, steps, warmup=1):
 
 def mfma_ceiling_leg(dev):
     """What a loop of nothing but MFMAs sustains on THIS box, in this process, after the timed region: the three MFMA
-    shapes (bf16 32x32x16 = the attention kernels' instruction, bf16 16x16x32, fp8 32x32x64) on all-zero operands and
+    shapes (bf16 16x16x32 = the bounded-score attention kernel's instruction, bf16 32x32x16, fp8 32x32x64 = the fp8
+    kernel's, fp8 16x16x128) on all-zero operands and
     on operands drawn from N(0, 1) activations (bf16) / their e4m3 quantisation (fp8), one wave per SIMD, ~30 ms
     launches, with the shader clock and the socket power sampled while each runs.  The part is power limited: the
     random-operand rate, not the 2.4 GHz figure, is what a kernel made of these MFMAs can reach here.
@@ -439,19 +460,23 @@ def mfma_ceiling_leg(dev):
     words_fp8 = (x * (448.0 / x.abs().max())).to(torch.float8_e4m3fn).view(torch.int32)  # 2^20 words of four e4m3 values
     sink = torch.empty(256 * 256, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    out = {"what": "MFMA-only loop, one wave per SIMD, operands in registers, 6 launches of ~30 ms after a warm-up; "
+    out = {"what": "MFMA-only loop, one wave per SIMD, operands in registers, launches of ~30 ms back to back after a warm-up "
+                   "(6 on zero operands, 30 on random ones; clock and power: median of the last 40 % of the samples); "
                    "random = N(0,1) activations as bf16 / as e4m3 scaled to absmax 448",
            "unit": "TFLOP/s"}
-    for name, kind, words in (("bf16_32x32x16", 0, words_bf16), ("bf16_16x16x32", 1, words_bf16), ("fp8_32x32x64", 2, words_fp8)):
+    for name, kind, words in (("bf16_32x32x16", 0, words_bf16), ("bf16_16x16x32", 1, words_bf16), ("fp8_32x32x64", 2, words_fp8),
+                              ("fp8_16x16x128", 3, words_fp8)):
         entry = {}
         for label, ptr in (("zero_operands", None), ("random_operands", words.data_ptr())):
             ms, fl = C.c_float(0), C.c_double(0)
-            with ClockSampler(period=0.01) as smp:
-                rc = lib.magi_probe_mfma_only(kind, ptr, sink.data_ptr(), 24000, 6, stream, C.byref(ms), C.byref(fl))
+            # (random operands run for ~0.9 s so that the sampled clock and power are this loop's, not its predecessor's)
+            with ClockSampler(period=0.02) as smp:
+                rc = lib.magi_probe_mfma_only(kind, ptr, sink.data_ptr(), 24000, 6 if ptr is None else 30, stream,
+                                              C.byref(ms), C.byref(fl))
             if rc != 0:
                 entry[label] = {"error": rc}
                 continue
-            clk, pw, _ = smp.result()
+            clk, pw, _ = smp.result(last_fraction=0.4)
             entry[label] = {"tflops": round(fl.value / (ms.value * 1e-3) / 1e12, 1), "ms_per_launch": round(ms.value, 2),
                             "shader_clock_mhz": None if clk is None else round(clk), "socket_power_w": None if pw is None else round(pw)}
         out[name] = entry
@@ -635,7 +660,7 @@ def main():
         ceil = mfma_ceiling_leg(dev)
         result["mfma_ceiling"] = ceil
         try:
-            top = ceil["bf16_32x32x16"]["random_operands"]["tflops"]
+            top = ceil["bf16_16x16x32"]["random_operands"]["tflops"]  # (the MFMA shape the core kernel is made of)
             result["roofline"]["measured_ceiling"] = top
             result["roofline"]["frac_of_measured_ceiling"] = round(core_tflops / top, 4)
             if "fp8" in result:

@@ -302,6 +302,19 @@ int magi_layer_norm(const void* x, int64_t x_stride, const void* weight, const v
                     void* y, int64_t y_stride, int64_t rows, int32_t cols, float eps, void* stream);
 
 /*
+ * The input quantiser of the reference's fp8 linear layers:
+ *     y = e4m3fn( bf16( clamp( float(x) / scale, -448, 448 ) ) )
+ * including the rounding to bf16 in the middle, which is part of the definition (a value may land on another e4m3
+ * code than a direct conversion would give).  Stands in for div_clamp_to (inference/model/dit/dit_module.py:364-384)
+ * as PerTensorQuantizedFp8Linear.forward applies it to the normalised hidden states ahead of bmm_fp8 (:445-456; the
+ * q, qx, k and v projections of every layer but the first and the last under fp8_quant, :405-409).
+ * x [rows, cols] bf16, y [rows, cols] e4m3 (row strides in elements); scale: DEVICE fp32, scale_len 1 (one value) or
+ * cols (one per column).  cols a multiple of 8.
+ */
+int magi_div_clamp_to_e4m3(const void* x, int64_t x_stride, const float* scale, int32_t scale_len, void* y,
+                           int64_t y_stride, int64_t rows, int32_t cols, void* stream);
+
+/*
  * Per-head norm only (no rotary, no cache): x [S, H, D] bf16 -> y [S, H, D] bf16, computed in the
  * precision the reference uses for the cross-attention norms (bf16 in, fp32 statistics, bf16 out).
  * Stands in for q_layernorm_xattn / k_layernorm_xattn in get_xqkv (dit_module.py:1008, 1020).

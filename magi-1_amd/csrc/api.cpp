@@ -399,6 +399,26 @@ int magi_layer_norm(const void* x, int64_t x_stride, const void* weight, const v
   return MAGI_OK;
 }
 
+int magi_div_clamp_to_e4m3(const void* x, int64_t x_stride, const float* scale, int32_t scale_len, void* y,
+                           int64_t y_stride, int64_t rows, int32_t cols, void* stream) {
+  if (rows < 0 || cols < 0) return fail(MAGI_EINVAL, "magi_div_clamp_to_e4m3: negative size");
+  if (rows == 0 || cols == 0) return MAGI_OK;
+  if (cols % 8) return fail(MAGI_ENOSYS, "magi_div_clamp_to_e4m3: cols %d is not a multiple of 8", cols);
+  if (!x || !y || !scale) return fail(MAGI_EINVAL, "magi_div_clamp_to_e4m3: NULL pointer");
+  if (scale_len != 1 && scale_len != cols)
+    return fail(MAGI_EINVAL, "magi_div_clamp_to_e4m3: scale_len %d (1, or cols = %d)", scale_len, cols);
+  if (x_stride < cols || y_stride < cols) return fail(MAGI_EINVAL, "magi_div_clamp_to_e4m3: row stride below cols");
+  if (x_stride % 8 || y_stride % 8 || !aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 7u) || !aligned16(scale))
+    return fail(MAGI_EINVAL, "magi_div_clamp_to_e4m3: rows of x must be 16-byte aligned, rows of y 8-byte, scale 16-byte");
+  if (rows * (int64_t)(cols / 8) > 0x7fffffffLL * 256)
+    return fail(MAGI_ENOSYS, "magi_div_clamp_to_e4m3: more than 2^39 groups of eight elements");
+  hipError_t e = magi::launch_div_clamp(static_cast<const char*>(x), x_stride * 2, scale, scale_len != 1,
+                                        static_cast<char*>(y), y_stride, rows, cols, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return hip_fail(e, "magi_div_clamp_to_e4m3 launch");
+  g_launches.fetch_add(1, std::memory_order_relaxed);
+  return MAGI_OK;
+}
+
 int magi_head_norm(const void* x, int64_t x_stride_t, int64_t x_stride_h, const float* gamma, const float* beta,
                    void* y, int32_t S, int32_t H, int32_t D, int32_t norm_kind, float eps, void* stream) {
   if (D != 128) return fail(MAGI_ENOSYS, "magi_head_norm: head_dim %d not implemented (128 only)", D);

@@ -105,6 +105,9 @@ hipError_t launch_head_norm(const char* x, long x_stride_t, long x_stride_h, con
                             char* y, int S, int H, int norm_kind, float eps, hipStream_t stream);
 hipError_t launch_layer_norm(const char* x, long x_stride, const void* w, const void* b, int params_fp32, char* y,
                              long y_stride, long rows, int cols, float eps, hipStream_t stream);
+// y = e4m3(bf16(clamp(x / scale, +-448))): x [rows, cols] bf16, y [rows, cols] e4m3, strides in BYTES
+hipError_t launch_div_clamp(const char* x, long x_stride, const float* scale, int per_column, char* y, long y_stride,
+                            long rows, int cols, hipStream_t stream);
 hipError_t launch_rotary(const void* x, const float* cos, const float* sin, void* y, int B, int S, int H, int D,
                          int R2, int is_bf16, hipStream_t stream);
 // Rows below n_first go to y / scales, the rest (row index and chunk index counted from n_first, a multiple of

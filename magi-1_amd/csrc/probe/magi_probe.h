@@ -8,7 +8,7 @@ extern "C" {
 #endif
 #define MAGI_PROBE_WORKGROUPS 256   /* one wave per SIMD on 256 CUs */
 #define MAGI_PROBE_SINK_FLOATS (MAGI_PROBE_WORKGROUPS * 256)
-/* kind 0: bf16 32x32x16, 1: bf16 16x16x32, 2: fp8 (e4m3) 32x32x64.
+/* kind 0: bf16 32x32x16, 1: bf16 16x16x32, 2: fp8 (e4m3) 32x32x64, 3: fp8 (e4m3) 16x16x128.
  * operands: DEVICE array of 2^20 32-bit words the MFMA operands are drawn from (random bit patterns of the
  *           operand type), or NULL for all-zero operands.  sink: DEVICE float[MAGI_PROBE_SINK_FLOATS].
  * Runs one warm-up launch and `launches` timed launches of `rounds` loop rounds back to back on `stream`, waits for

@@ -37,6 +37,7 @@ constexpr int OPERAND_WORDS = 1 << 20;
 // KIND 0: v_mfma_f32_32x32x16_bf16 (the attention kernels' MFMA), 64 per round over 8 accumulators
 // KIND 1: v_mfma_f32_16x16x32_bf16, 128 per round over 16 accumulators (the same FLOPs per round)
 // KIND 2: v_mfma_scale_f32_32x32x64_f8f6f4 on e4m3 operands (the fp8 kernel's MFMA), 32 per round over 8 accumulators
+// KIND 3: v_mfma_scale_f32_16x16x128_f8f6f4 on e4m3 operands, 64 per round over 16 accumulators (the same FLOPs)
 template <int KIND>
 __global__ __launch_bounds__(256, 1) void mfma_only_kernel(const uint32_t* operands, float* sink, int rounds) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
@@ -49,7 +50,23 @@ __global__ __launch_bounds__(256, 1) void mfma_only_kernel(const uint32_t* opera
       rb[j][v] = operands ? operands[(t * 131 + j * 8 + v + 4) & (OPERAND_WORDS - 1)] : 0u;
     }
   float r = 0.f;
-  if constexpr (KIND == 1) {
+  if constexpr (KIND == 3) {
+    f32x4 acc[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int it = 0; it < rounds; ++it) {
+      static_for<0, 64>([&](auto sc) __attribute__((always_inline)) {
+        constexpr int s = decltype(sc)::value;
+        acc[s & 15] = __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(*(i32x8*)ra[s & 7], *(i32x8*)rb[(s >> 3) & 7], acc[s & 15],
+                                                                       0, 0, 0, 0, 0, 0);
+      });
+      if ((it & 63) == 63)
+#pragma unroll
+        for (int j = 0; j < 16; ++j) acc[j] *= 1e-3f;
+    }
+#pragma unroll
+    for (int j = 0; j < 16; ++j) r += acc[j][0] + acc[j][1] + acc[j][2] + acc[j][3];
+  } else if constexpr (KIND == 1) {
     f32x4 acc[16];
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[j] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -100,7 +117,7 @@ __global__ __launch_bounds__(256, 1) void mfma_only_kernel(const uint32_t* opera
 
 extern "C" int magi_probe_mfma_only(int kind, const uint32_t* operands, float* sink, int rounds, int launches,
                                     void* stream, float* ms_per_launch, double* flop_per_launch) {
-  if (kind < 0 || kind > 2 || !sink || rounds <= 0 || launches <= 0 || !ms_per_launch || !flop_per_launch) return -22;
+  if (kind < 0 || kind > 3 || !sink || rounds <= 0 || launches <= 0 || !ms_per_launch || !flop_per_launch) return -22;
   hipStream_t st = static_cast<hipStream_t>(stream);
   hipEvent_t e0, e1;
   if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) return -5;
@@ -109,6 +126,7 @@ extern "C" int magi_probe_mfma_only(int kind, const uint32_t* operands, float* s
     if (kind == 0) hipLaunchKernelGGL(mfma_only_kernel<0>, grid, block, 0, st, operands, sink, rounds);
     if (kind == 1) hipLaunchKernelGGL(mfma_only_kernel<1>, grid, block, 0, st, operands, sink, rounds);
     if (kind == 2) hipLaunchKernelGGL(mfma_only_kernel<2>, grid, block, 0, st, operands, sink, rounds);
+    if (kind == 3) hipLaunchKernelGGL(mfma_only_kernel<3>, grid, block, 0, st, operands, sink, rounds);
   };
   launch();  // warm-up, also brings the board to its operating point
   (void)hipEventRecord(e0, st);
@@ -121,8 +139,8 @@ extern "C" int magi_probe_mfma_only(int kind, const uint32_t* operands, float* s
   (void)hipEventDestroy(e1);
   if (e != hipSuccess || hipGetLastError() != hipSuccess) return -5;
   *ms_per_launch = ms / launches;
-  // per round and wave: 64 x 32x32x16 = 128 x 16x16x32 = 32 x 32x32x64 (fp8: twice the FLOPs of the bf16 round)
-  const double per_round = (kind == 2 ? 2.0 : 1.0) * 64.0 * 2.0 * 32 * 32 * 16;
+  // per round and wave: 64 x 32x32x16 = 128 x 16x16x32; 32 x 32x32x64 = 64 x 16x16x128 (fp8: twice the FLOPs)
+  const double per_round = (kind >= 2 ? 2.0 : 1.0) * 64.0 * 2.0 * 32 * 32 * 16;
   *flop_per_launch = per_round * rounds * MAGI_PROBE_WORKGROUPS * 4.0;
   return 0;
 }

@@ -356,7 +356,58 @@ __global__ __launch_bounds__(THREADS) void rotary_kernel(const void* xin, const 
   }
 }
 
+// div_clamp_to: y = e4m3(bf16(clamp(float(x) / scale, -448, 448))), the fp8 linears' input quantiser with its bf16
+// intermediate (a double rounding that is part of the definition).  One thread per 8 consecutive elements of a row;
+// scale: one value, or one per column.  IEEE division (the reference divides in fp32).
+__global__ __launch_bounds__(THREADS) void div_clamp_kernel(const char* x, long xs, const float* scale, int per_column,
+                                                            char* y, long ys, long rows, int cols8) {
+  const long t = (long)blockIdx.x * THREADS + threadIdx.x;
+  if (t >= rows * cols8) return;
+  const long r = t / cols8;
+  const int c = (int)(t - r * cols8);
+  float f[8];
+  unpack8(*(const u32x4*)(x + r * xs + (long)c * 16), f);
+  float sc[8];
+  if (per_column) {
+    const f32x4 s0 = *(const f32x4*)(scale + 8 * c), s1 = *(const f32x4*)(scale + 8 * c + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      sc[i] = s0[i];
+      sc[4 + i] = s1[i];
+    }
+  } else {
+    const float s = scale[0];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) sc[i] = s;
+  }
+  float q[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const float d = f[i] / sc[i];
+    const float cl = d != d ? d : fminf(fmaxf(d, -448.f), 448.f);  // (a NaN stays a NaN, as torch.clamp leaves it)
+    q[i] = (float)(__bf16)cl;                                     // the bf16 intermediate
+  }
+  u32x2 o;
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    int u = 0;
+    u = __builtin_amdgcn_cvt_pk_fp8_f32(q[4 * j], q[4 * j + 1], u, false);
+    u = __builtin_amdgcn_cvt_pk_fp8_f32(q[4 * j + 2], q[4 * j + 3], u, true);
+    o[j] = (unsigned)u;
+  }
+  *(u32x2*)(y + r * ys + (long)c * 8) = o;
+}
+
 }  // namespace
+
+hipError_t launch_div_clamp(const char* x, long x_stride, const float* scale, int per_column, char* y, long y_stride,
+                            long rows, int cols, hipStream_t stream) {
+  const long n = rows * (cols / 8);
+  if (n <= 0) return hipSuccess;
+  hipLaunchKernelGGL(div_clamp_kernel, dim3((unsigned)((n + THREADS - 1) / THREADS)), dim3(THREADS), 0, stream, x, x_stride,
+                     scale, per_column, y, y_stride, rows, cols / 8);
+  return hipGetLastError();
+}
 
 hipError_t launch_prologue(const PrologueKernArgs& a_in, hipStream_t stream) {
   if (a_in.S <= 0) return hipSuccess;

@@ -106,7 +106,7 @@ class QuantizeArgs(_SizedStructure):
 ABI_VERSION = 102  # magi_version() of the library these mirrors were written for
 
 EXPORTS = ("magi_version", "magi_last_error", "magi_launch_count", "magi_attn_fwd", "magi_qk_prologue", "magi_head_norm",
-           "magi_apply_rotary", "magi_quantize_fp8", "magi_quantize_fp8_split", "magi_layer_norm", "magi_qkv_proj_prologue")
+           "magi_apply_rotary", "magi_quantize_fp8", "magi_quantize_fp8_split", "magi_layer_norm", "magi_qkv_proj_prologue", "magi_div_clamp_to_e4m3")
 
 _lib = None
 
@@ -136,6 +136,9 @@ def lib() -> C.CDLL:
         l.magi_layer_norm.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_void_p, C.c_int32, C.c_void_p, C.c_int64,
                                       C.c_int64, C.c_int32, C.c_float, C.c_void_p]
         l.magi_layer_norm.restype = C.c_int
+        l.magi_div_clamp_to_e4m3.argtypes = [C.c_void_p, C.c_int64, C.c_void_p, C.c_int32, C.c_void_p, C.c_int64, C.c_int64,
+                                             C.c_int32, C.c_void_p]
+        l.magi_div_clamp_to_e4m3.restype = C.c_int
         l.magi_apply_rotary.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_int32,
                                         C.c_int32, C.c_int32, C.c_int32, C.c_int32, C.c_void_p]
         l.magi_apply_rotary.restype = C.c_int

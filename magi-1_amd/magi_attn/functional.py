@@ -485,6 +485,31 @@ def layer_norm(x: torch.Tensor, weight: Optional[torch.Tensor], bias: Optional[t
     return y
 
 
+def div_clamp_to(x: torch.Tensor, scale: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """e4m3fn(bf16(clamp(x.float() / scale.float(), -448, 448))): the input quantiser of the reference's fp8 linears
+    (dit_module.py:364-384), double rounding included.  x: bf16, last axis contiguous (leading axes collapsible to one
+    row stride); scale: fp32 with one element or one per element of the last axis.  -> float8_e4m3fn, x's shape."""
+    if x.dtype != torch.bfloat16:
+        raise TypeError("x must be bf16")
+    if not x.is_cuda:
+        raise ValueError("x must be a device tensor (there is no CPU path)")
+    cols = x.shape[-1]
+    x2 = x if x.dim() == 2 else x.reshape(-1, cols)
+    if x2.stride(-1) != 1:
+        x2 = x2.contiguous()
+    sc = scale.detach().to(device=x.device, dtype=torch.float32).reshape(-1).contiguous()
+    if sc.numel() not in (1, cols):
+        raise ValueError("scale must have one element, or one per element of x's last axis")
+    y = torch.empty(x.shape, dtype=torch.float8_e4m3fn, device=x.device) if out is None else out
+    if y.shape != x.shape or y.dtype != torch.float8_e4m3fn or y.device != x.device or not y.is_contiguous():
+        raise ValueError("out must be a contiguous float8_e4m3fn tensor of x's shape on x's device")
+    rows = x2.shape[0]
+    with torch.cuda.device(x.device):
+        L.check(L.lib().magi_div_clamp_to_e4m3(x2.data_ptr(), x2.stride(0) if rows > 1 else cols, sc.data_ptr(), sc.numel(),
+                                               y.data_ptr(), cols, rows, cols, _stream()))
+    return y
+
+
 def head_norm(x: torch.Tensor, gamma, beta, eps: float = 1e-6, norm_kind: int = L.MAGI_NORM_LAYERNORM_1P):
     """x [S, H, 128] bf16 (strided heads allowed) -> contiguous normalised copy."""
     _check_thd(x, "x")

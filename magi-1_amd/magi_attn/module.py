@@ -32,7 +32,7 @@ import math
 
 from . import _lib as L
 from .cache import Fp8KVCache
-from .functional import (head_norm, layer_norm, pow2_scale_for, qk_prologue, qk_prologue_fp8, qkv_proj_prologue,
+from .functional import (div_clamp_to, head_norm, layer_norm, pow2_scale_for, qk_prologue, qk_prologue_fp8, qkv_proj_prologue,
                          quantize_fp8_split,
                          range_attention)
 from .params import InferenceParams, ModelMetaArgs, PackedCrossAttnParams
@@ -133,8 +133,50 @@ def qk_score_bound(q_norm: FusedLayerNorm, k_norm: FusedLayerNorm, rotary_half: 
     return float(bound.item())
 
 
+class PerTensorQuantizedFp8Linear(torch.nn.Module):
+    """The reference's fp8 linear layer (dit_module.py:431-456) with its parameter names and shapes, so that its
+    checkpoints load: `weight` [1, out, in] float8_e4m3fn, `weight_scale` [1] fp32, `input_scale` [in] fp32.
+
+    forward: x8 = div_clamp_to(x, input_scale) (magi_div_clamp_to_e4m3: the reference's quantiser, bf16 intermediate
+    included), then the library's fp8 GEMM with fp32 accumulation, de-quantised by input_scale * weight_scale, bf16
+    out (the reference calls flashinfer's bmm_fp8, which reads ONE value behind each scale pointer: with the
+    per-channel shape the reference gives input_scale, that is its first element, as here).  The GEMM itself is
+    a library routine (hipBLASLt through torch._scaled_mm), like the bf16 projections'."""
+
+    def __init__(self, in_features: int, out_features: int, bias=False, dtype=torch.bfloat16, device=None) -> None:
+        super().__init__()
+        self.in_features, self.out_features, self.output_dtype = in_features, out_features, dtype
+        P_ = torch.nn.Parameter
+        self.weight = P_(torch.zeros((1, out_features, in_features), device=device).to(torch.float8_e4m3fn), requires_grad=False)
+        self.weight_scale = P_(torch.ones(1, dtype=torch.float32, device=device), requires_grad=False)
+        self.input_scale = P_(torch.ones(in_features, dtype=torch.float32, device=device), requires_grad=False)
+
+    @classmethod
+    def from_linear(cls, lin: torch.nn.Linear, input_absmax: float) -> "PerTensorQuantizedFp8Linear":
+        """Per-tensor quantisation of a bf16 linear layer (for tests and calibration scripts): weight scale from the
+        weight's absmax, input scale from the given absmax of the inputs, both so that the maximum maps to 448."""
+        w = lin.weight.detach().float()
+        q = cls(lin.in_features, lin.out_features, dtype=lin.weight.dtype, device=w.device)
+        ws = (w.abs().max() / 448.0).clamp_min(1e-12)
+        q.weight.data = (w / ws).clamp(-448, 448).to(torch.float8_e4m3fn)[None]
+        q.weight_scale.data = ws.reshape(1).float()
+        q.input_scale.data = torch.full((lin.in_features,), float(input_absmax) / 448.0, dtype=torch.float32, device=w.device)
+        return q
+
+    def forward(self, input: torch.Tensor) -> torch.Tensor:
+        x8 = div_clamp_to(input, self.input_scale)
+        prefix = input.shape[:-1]
+        y = torch._scaled_mm(x8.reshape(-1, self.in_features), self.weight[0].t(), scale_a=self.input_scale.reshape(-1)[:1],
+                             scale_b=self.weight_scale.reshape(-1)[:1], out_dtype=self.output_dtype)
+        return y.reshape(prefix + (self.out_features,))
+
+
 class CustomLayerNormLinear(torch.nn.Module):
     """Input LayerNorm + the four projections q, qx, k, v (dit_module.py:390-425).
+
+    fp8_quant=True builds the four projections as PerTensorQuantizedFp8Linear, as the reference does for every
+    layer but the first and the last under EngineConfig.fp8_quant (:405-409): each quantises the normalised input
+    with its own input scale and runs the library's fp8 GEMM; there is no shared weight buffer then.
 
     The four weights keep the reference's parameter names (q.weight, qx.weight, k.weight, v.weight) but live
     side by side in ONE buffer, rows ordered [q | k | v | qx], so forward_qkvx() is a single GEMM over the
@@ -144,14 +186,15 @@ class CustomLayerNormLinear(torch.nn.Module):
     next call."""
 
     def __init__(self, input_size: int, output_size_q: int, output_size_kv: int, eps: float = 1e-6,
-                 dtype=torch.bfloat16, device=None):
+                 dtype=torch.bfloat16, device=None, fp8_quant: bool = False):
         super().__init__()
+        self.fp8_quant = bool(fp8_quant)
         self.layer_norm = torch.nn.LayerNorm(input_size, eps=eps, dtype=dtype, device=device)
-        self.q = torch.nn.Linear(input_size, output_size_q, bias=False, dtype=dtype, device=device)
-        self.qx = torch.nn.Linear(input_size, output_size_q, bias=False, dtype=dtype, device=device)
-        self.k = torch.nn.Linear(input_size, output_size_kv, bias=False, dtype=dtype, device=device)
-        self.v = torch.nn.Linear(input_size, output_size_kv, bias=False, dtype=dtype, device=device)
-        self._fuse_weights()
+        mk = (lambda n: PerTensorQuantizedFp8Linear(input_size, n, dtype=dtype, device=device)) if self.fp8_quant else \
+            (lambda n: torch.nn.Linear(input_size, n, bias=False, dtype=dtype, device=device))
+        self.q, self.qx, self.k, self.v = mk(output_size_q), mk(output_size_q), mk(output_size_kv), mk(output_size_kv)
+        if not self.fp8_quant:
+            self._fuse_weights()
 
     def _projections(self):
         return (self.q, self.k, self.v, self.qx)  # row order of the shared buffer
@@ -183,7 +226,9 @@ class CustomLayerNormLinear(torch.nn.Module):
 
     def forward_qkvx(self, hidden_states):
         """One GEMM for all four projections of the (already normalised) input -> views (q, k, v, qx) of one
-        [..., 2*out_q + 2*out_kv] result."""
+        [..., 2*out_q + 2*out_kv] result.  (fp8_quant: four quantise + fp8 GEMM pairs, each with its own scales.)"""
+        if self.fp8_quant:
+            return self.q(hidden_states), self.k(hidden_states), self.v(hidden_states), self.qx(hidden_states)
         y = torch.nn.functional.linear(hidden_states, self.fused_weight())
         oq, okv = self.q.weight.shape[0], self.k.weight.shape[0]
         return y[..., :oq], y[..., oq:oq + okv], y[..., oq + okv:oq + 2 * okv], y[..., oq + 2 * okv:]
@@ -211,13 +256,15 @@ class FullyParallelAttention(torch.nn.Module):
     def __init__(self, hidden_size: int, num_attention_heads: int, num_query_groups: int, kv_channels: int = 128,
                  layer_number: int = 0, layernorm_epsilon: float = 1e-6, apply_layernorm_1p: bool = True,
                  xattn_cond_hidden_ratio: float = 1.0, params_dtype=torch.bfloat16, device=None,
-                 attention_dtype: str = "bf16", fp8_fast_exp2: bool = False, fused_projection: bool = False):
+                 attention_dtype: str = "bf16", fp8_fast_exp2: bool = False, fused_projection: bool = False,
+                 fp8_quant: bool = False):
         """attention_dtype "fp8" (not in the reference, which has no fp8 attention) runs the self-attention on
         e4m3 operands with per-(video chunk, head) power-of-two scales and keeps the KV cache in that form
         (Fp8KVCache); the cross attention and everything else stay in bf16.
         fp8_fast_exp2: False (default) = the exact exponential, "softmax in fp32"; True opts into the fp8 kernel's
         piecewise-linear exp2 (MAGI_ATTN_FP8_FAST_EXP2: about 15 % faster, probabilities up to 6.2 % off each, the
         output inside a looser accuracy bar; see include/magi_attn.h).
+        fp8_quant: the q / qx / k / v projections as PerTensorQuantizedFp8Linear (the reference's fp8_quant layers).
         fused_projection: run the four projections and the prologue as ONE launch (magi_qkv_proj_prologue, the
         hand-written GEMM whose epilogue is the prologue) instead of a library GEMM followed by the prologue kernel;
         bf16 attention at batch 1 only.  Off by default: at the 720p shape the library GEMM + prologue take
@@ -229,7 +276,7 @@ class FullyParallelAttention(torch.nn.Module):
             raise ValueError("attention_dtype must be 'bf16' or 'fp8'")
         self.attention_dtype = attention_dtype
         self.fp8_fast_exp2 = bool(fp8_fast_exp2)
-        self.fused_projection = bool(fused_projection)
+        self.fused_projection = bool(fused_projection) and not fp8_quant
         # forward() has the prologue fold softmax_scale * log2(e) into q ahead of q's one rounding to bf16 and tells
         # the attention kernel so (no per-score multiply there); get_q / get_qkv return q unscaled, as the reference
         self._q_premul = kv_channels ** -0.5 * math.log2(math.e)
@@ -241,7 +288,7 @@ class FullyParallelAttention(torch.nn.Module):
         self.kv_projection_size = kv_channels * num_query_groups
         self.eps = layernorm_epsilon
         self.linear_qkv = CustomLayerNormLinear(hidden_size, self.query_projection_size, self.kv_projection_size,
-                                                eps=layernorm_epsilon, dtype=params_dtype, device=device)
+                                                eps=layernorm_epsilon, dtype=params_dtype, device=device, fp8_quant=fp8_quant)
         self.linear_kv_xattn = torch.nn.Linear(int(hidden_size * xattn_cond_hidden_ratio), 2 * self.kv_projection_size,
                                                bias=False, dtype=params_dtype, device=device)
         mk = lambda dt: FusedLayerNorm(kv_channels, layernorm_epsilon, apply_layernorm_1p, dtype=dt, device=device)

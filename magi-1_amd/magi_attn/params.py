@@ -61,6 +61,23 @@ class InferenceParams:
         self.key_value_memory_dict = {}
         self.update_kv_cache = False
 
+    def swap_key_value_dict(self, batch_idx):
+        """Re-order the batch rows of every layer's cache (dataclass.py:72-83).  The reference's method is written
+        for a (key, value) tuple of [seq, batch, ...] tensors, a layout its DiT never stores (its caches are the
+        single [max_seq * max_bs, Hkv, 2D] tensors of dit_module.py:800-819, tokens ordered (position, batch)), and
+        the shipped pipeline never calls it; this one does the same thing on the layout that is actually used.
+        Raises on an empty dict like the reference."""
+        if len(self.key_value_memory_dict) == 0:
+            raise ValueError("should not swap when dict in empty")
+        idx = torch.as_tensor(batch_idx, dtype=torch.long)
+        if idx.numel() != self.max_batch_size:
+            raise ValueError("batch_idx must name every batch row once")
+        for layer_number, cache in self.key_value_memory_dict.items():
+            if not isinstance(cache, torch.Tensor):
+                raise TypeError("swap_key_value_dict works on tensor caches (not on an Fp8KVCache)")
+            rows = cache.view(self.max_sequence_length, self.max_batch_size, *cache.shape[1:])
+            self.key_value_memory_dict[layer_number] = rows[:, idx.to(cache.device)].reshape(cache.shape)
+
 
 def build_core_attn_params(q_range: torch.Tensor, k_range: torch.Tensor, max_seqlen_q: int,
                            max_seqlen_k: Optional[int] = None) -> PackedCoreAttnParams:

@@ -309,3 +309,21 @@ def test_attention_kernels_keep_their_registers():
                 assert sc <= limit, f"{n}: {sc} bytes of scratch per lane"
                 assert vg <= 256
         assert seen >= 2
+
+
+def test_inference_params_swap_key_value_dict():
+    """Batch rows of the (position, batch)-ordered caches are re-ordered in every layer; an empty dict raises, as in
+    the reference (inference/common/dataclass.py:72-83)."""
+    from magi_attn.params import InferenceParams
+
+    ip = InferenceParams(3, 4)
+    with pytest.raises(ValueError):
+        ip.swap_key_value_dict([0, 1, 2])
+    c = torch.arange(4 * 3 * 2 * 8, dtype=torch.float32).view(12, 2, 8)  # [max_seq * max_bs, Hkv, 2D]
+    ip.key_value_memory_dict[0] = c.clone()
+    ip.key_value_memory_dict[5] = c.clone() + 1000
+    ip.swap_key_value_dict([2, 0, 1])
+    want = c.view(4, 3, 2, 8)[:, [2, 0, 1]].reshape(12, 2, 8)
+    assert torch.equal(ip.key_value_memory_dict[0], want) and torch.equal(ip.key_value_memory_dict[5], want + 1000)
+    with pytest.raises(ValueError):
+        ip.swap_key_value_dict([0, 1])

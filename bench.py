@@ -37,8 +37,8 @@ SCORE_BOUND = 1.01 * 128 * Q_PREMUL
 # HBM-side bytes per launch on the 720p workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a
 # plain copy of known size in the same run (both counters read 1.00 x the bytes of the copy).  NOT measured in this run:
 # the figures and the commands that produced them are in profiles/bench_720p_hbm_traffic_pmc.txt
-MEASURED_TRAFFIC = {"720p-24B": {"core": 70.25e9 + 1.06e9, "prologue": 0.724e9 + 1.4385e9,
-                                 "layer_norm": 0.531e9 + 1.0617e9, "cross": 0.722e9 + 1.379e9}}
+MEASURED_TRAFFIC = {"720p-24B": {"core": 105.45e9 + 1.0617e9, "prologue": 0.7245e9 + 1.4367e9,
+                                 "layer_norm": 0.531e9 + 1.0617e9, "cross": 0.5673e9 + 1.0617e9}}
 TRAFFIC_SOURCE = "profiles/bench_720p_hbm_traffic_pmc.txt (counter run of this command, not this run)"
 
 
@@ -460,8 +460,9 @@ def mfma_ceiling_leg(dev):
     words_fp8 = (x * (448.0 / x.abs().max())).to(torch.float8_e4m3fn).view(torch.int32)  # 2^20 words of four e4m3 values
     sink = torch.empty(256 * 256, device=dev)
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    out = {"what": "MFMA-only loop, one wave per SIMD, operands in registers, launches of ~30 ms back to back after a warm-up "
-                   "(6 on zero operands, 30 on random ones; clock and power: median of the last 40 % of the samples); "
+    out = {"what": "MFMA-only loop, one wave per SIMD, operands in registers, 100 launches of 20-30 ms back to back after a "
+                   "warm-up (2-3 s per entry: the socket power the driver reports is an average over about a second; clock "
+                   "and power: median of the last 30 % of the samples); "
                    "random = N(0,1) activations as bf16 / as e4m3 scaled to absmax 448",
            "unit": "TFLOP/s"}
     for name, kind, words in (("bf16_32x32x16", 0, words_bf16), ("bf16_16x16x32", 1, words_bf16), ("fp8_32x32x64", 2, words_fp8),
@@ -469,14 +470,14 @@ def mfma_ceiling_leg(dev):
         entry = {}
         for label, ptr in (("zero_operands", None), ("random_operands", words.data_ptr())):
             ms, fl = C.c_float(0), C.c_double(0)
-            # (random operands run for ~0.9 s so that the sampled clock and power are this loop's, not its predecessor's)
+            # (2-3 s per entry so that the sampled clock and power are this loop's, not its predecessor's)
             with ClockSampler(period=0.02) as smp:
-                rc = lib.magi_probe_mfma_only(kind, ptr, sink.data_ptr(), 24000, 6 if ptr is None else 30, stream,
+                rc = lib.magi_probe_mfma_only(kind, ptr, sink.data_ptr(), 24000, 100, stream,
                                               C.byref(ms), C.byref(fl))
             if rc != 0:
                 entry[label] = {"error": rc}
                 continue
-            clk, pw, _ = smp.result(last_fraction=0.4)
+            clk, pw, _ = smp.result(last_fraction=0.3)
             entry[label] = {"tflops": round(fl.value / (ms.value * 1e-3) / 1e12, 1), "ms_per_launch": round(ms.value, 2),
                             "shader_clock_mhz": None if clk is None else round(clk), "socket_power_w": None if pw is None else round(pw)}
         out[name] = entry

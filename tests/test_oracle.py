@@ -400,6 +400,25 @@ def test_fp8_quantiser_properties():
     assert t8.float().abs().max() == 448  # absmax maps onto the top code
 
 
+def test_div_clamp_double_rounding_through_bf16_hand_computed():
+    """The reference's linear-layer quantiser rounds x / scale to bf16 before e4m3 (dit_module.py:376-381).  e4m3 has
+    a grid of 1/8 in [1, 2) and bf16 one of 1/128, so a value just beside an e4m3 midpoint first lands ON the midpoint
+    and then goes to the even code: worked out by hand, and different from the single rounding in both directions."""
+    up = 1.0625 + 2.0 ** -10     # above the midpoint of 1.0 and 1.125: one rounding gives 1.125
+    down = 1.1875 - 2.0 ** -10   # below the midpoint of 1.125 and 1.25: one rounding gives 1.125
+    x = torch.tensor([up, down, -up, -down, 3.0 * up, 1e9, -1e9])
+    one = O.quantize_e4m3(x, torch.tensor(1.0)).float()
+    two = O.quantize_e4m3(x, torch.tensor(1.0), via_bf16=True).float()
+    assert one.tolist() == [1.125, 1.125, -1.125, -1.125, 3.25, 448.0, -448.0]
+    # bf16 first: 1.0625 exactly (tie -> even mantissa 000 = 1.0), 1.1875 exactly (tie -> even mantissa 010 = 1.25);
+    # 3 x up = 3.189 is nearer 3.25 than 3.0 (grid 1/4 in [2, 4)) with either rounding
+    assert two.tolist() == [1.0, 1.25, -1.0, -1.25, 3.25, 448.0, -448.0]
+    # the scale divides first: the same codes from 4 x the values with scale 4, and per-column scales broadcast
+    assert O.quantize_e4m3(4.0 * x, torch.tensor(4.0), via_bf16=True).float().tolist() == two.tolist()
+    cols = O.quantize_e4m3(torch.tensor([[up, 2.0 * up]]), torch.tensor([1.0, 2.0]), via_bf16=True).float()
+    assert cols.tolist() == [[1.0, 1.0]]
+
+
 def test_prologue_premul_is_the_softmax_scale_moved_into_q():
     """prologue(q_premul=c) has no counterpart in the reference.  Pin: with c = softmax_scale * log2(e) the
     pre-scaled q through attention with softmax_scale = ln 2 equals (up to q's bf16 rounding) the reference-shaped

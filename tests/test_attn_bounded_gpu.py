@@ -120,6 +120,37 @@ def test_bounded_varlen_segments_with_empty_and_ragged_keys(dev):
     _cmp(out, ref)
 
 
+@pytest.mark.parametrize("mode", ["prescaled", "scale_on_load", "mfma32"])
+def test_bounded_every_key_tail_length(dev, mode):
+    """Key segments of every length from 1 to 131 in one launch (every position of the ragged end inside a 64-key
+    tile and inside its 16-key blocks, with one, two and three tiles), query segments of 3 to 67 rows (partly filled
+    16-row blocks and waves), an offset start of the key axis; output and lse against the oracle per segment."""
+    Hq, Hkv = 4, 2
+    k_lens = np.arange(1, 132)
+    q_lens = 3 + (np.arange(len(k_lens)) * 7) % 65
+    qs = np.concatenate([[0], np.cumsum(q_lens)])
+    ks = 5 + np.concatenate([[0], np.cumsum(k_lens)])       # keys start at row 5, not at a tile boundary
+    qr = np.stack([qs[:-1], qs[1:]], 1)
+    kr = np.stack([ks[:-1], ks[1:]], 1)
+    q, k, v, bound = _inputs(int(qs[-1]), int(ks[-1]) + 9, Hq, Hkv, seed=23)
+    tq, tk = _ranges(dev, qr, kr)
+    if mode == "scale_on_load":
+        q_in = (q.float() / PREMUL).bfloat16()                # unscaled q: the kernel applies softmax_scale * log2(e)
+        kw, scale = dict(score_bound=1.01 * bound), None      # (oracle: default softmax scale, natural exponential)
+    else:
+        q_in, scale = q, LN2
+        kw = dict(q_prescaled=True, score_bound=bound, bounded_mfma32=(mode == "mfma32"))
+    out, lse = M.range_attention(q_in.to(dev), k.to(dev), v.to(dev), tq, tk, int(q_lens.max()), int(k_lens.max()), **kw)
+    ref = O.range_attention(q_in, k, v, qr, kr, softmax_scale=scale)
+    ref_lse = O.range_attention_lse(q_in, k, v, qr, kr, softmax_scale=scale)
+    _cmp(out, ref, mode)
+    # (the lse of a one-key segment IS its score; the second rounding of q moves a score by ~2e-3 r.m.s., so the
+    # largest of 20000 rows lies around four times that)
+    assert (lse.cpu() - ref_lse).abs().max().item() < (2e-2 if mode == "scale_on_load" else 5e-3)
+    worst = max(((out[a:b].double().cpu() - ref[a:b].double()).abs().max().item(), int(n)) for (a, b), n in zip(qr, k_lens))
+    assert worst[0] <= MAX_ABS, f"segment with {worst[1]} keys: {worst[0]}"
+
+
 @pytest.mark.parametrize("mfma32", [False, True])
 def test_bounded_cache_views_two_segments_and_grouped_output(dev, mfma32):
     """K / V read in place from an interleaved cache, the key axis split into [cache prefix | side buffer] at

@@ -31,7 +31,7 @@ import torch
 import math
 
 from . import _lib as L
-from .cache import Fp8KVCache
+from .cache import Fp8KVCache, OffloadedKVCache
 from .functional import (div_clamp_to, head_norm, layer_norm, pow2_scale_for, qk_prologue, qk_prologue_fp8, qkv_proj_prologue,
                          quantize_fp8_split,
                          range_attention)
@@ -329,7 +329,8 @@ class FullyParallelAttention(torch.nn.Module):
 
     # ------------------------------------------------------------------ cache
     def _allocate_key_and_value_memory(self, sequence_length: int, batch_size: int, dtype) -> torch.Tensor:
-        """[max_seq * max_bs, Hkv, 2D] in HBM (dit_module.py:800-819; no pinned-host variant)."""
+        """[max_seq * max_bs, Hkv, 2D] in HBM (dit_module.py:800-819).  The pinned-host variant is not made here: a
+        KVCacheArena(kv_offload=True) attached to the InferenceParams supplies it for all layers."""
         return torch.empty(sequence_length * batch_size, self.num_query_groups_per_partition,
                            2 * self.hidden_size_per_attention_head, dtype=dtype,
                            device=self.linear_qkv.q.weight.device)
@@ -544,16 +545,24 @@ class FullyParallelAttention(torch.nn.Module):
         if meta_args.extract_prefix_video_feature or meta_args.fwd_extra_1st_chunk or meta_args.slice_point > 0:
             cache = self._cache(inference_params, key_and_value.dtype)
             start = meta_args.slice_point * meta_args.clip_token_nums * inference_params.max_batch_size
-            prefix = cache[:start]
-            if inference_params.update_kv_cache:
-                total = key_and_value.size(0)
-                clip = (total - meta_args.clip_token_nums * inference_params.max_batch_size
-                        if meta_args.distill_nearly_clean_chunk else total)
-                if start + clip > cache.size(0):
-                    raise ValueError("KV cache overflow")
-                prefix = prefix.clone()
-                cache[start:start + clip] = key_and_value[:clip]
-            key_and_value = torch.cat([prefix, key_and_value], dim=0)
+            offloaded = cache if isinstance(cache, OffloadedKVCache) else None
+            if offloaded is not None:
+                cache = offloaded.stage(start)
+            clip = 0
+            try:
+                prefix = cache[:start]
+                if inference_params.update_kv_cache:
+                    total = key_and_value.size(0)
+                    clip = (total - meta_args.clip_token_nums * inference_params.max_batch_size
+                            if meta_args.distill_nearly_clean_chunk else total)
+                    if start + clip > cache.shape[0]:
+                        clip = 0
+                        raise ValueError("KV cache overflow")
+                    cache[start:start + clip] = key_and_value[:clip]
+                key_and_value = torch.cat([prefix, key_and_value], dim=0)
+            finally:
+                if offloaded is not None:
+                    offloaded.release(start, clip)
         return key_and_value[..., :D].contiguous(), key_and_value[..., D:].contiguous()
 
     def core_attention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, bs: int,
@@ -714,11 +723,16 @@ class FullyParallelAttention(torch.nn.Module):
             cache = self._cache(inference_params, hidden_states.dtype)
             start = meta_args.slice_point * meta_args.clip_token_nums
             S = sq
+            offloaded = cache if isinstance(cache, OffloadedKVCache) else None
+            if offloaded is not None:  # kv_offload: the prefix comes through a device staging buffer
+                cache = offloaded.stage(start)
             if inference_params.update_kv_cache:
                 n_keep = S - meta_args.clip_token_nums if meta_args.distill_nearly_clean_chunk else S
             else:
                 n_keep = 0
             if start + n_keep > cache.shape[0]:
+                if offloaded is not None:
+                    offloaded.release()
                 raise ValueError("KV cache overflow")
             tail = None
             if n_keep < S:  # side buffer for the rows that must not be persisted, kept between calls
@@ -728,16 +742,22 @@ class FullyParallelAttention(torch.nn.Module):
                     tail = torch.empty(S - n_keep, cache.shape[1], cache.shape[2], dtype=cache.dtype, device=cache.device)
                     self._kv_tail = tail
                 tail = tail[:S - n_keep]
-            q, _, qx_raw = project(kv_out=cache[start:], n_cache_rows=n_keep, kv_tail=tail)
-            split = start + n_keep
-            kc, vc = cache[:split, :, :D], cache[:split, :, D:]
-            if tail is None:
-                core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                          out=core_dst, return_lse=False, q_prescaled=True, score_bound=bound_core)
-            else:
-                core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                          k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, out=core_dst,
-                                          return_lse=False, q_prescaled=True, score_bound=bound_core)
+            persisted = 0
+            try:
+                q, _, qx_raw = project(kv_out=cache[start:], n_cache_rows=n_keep, kv_tail=tail)
+                split = start + n_keep
+                kc, vc = cache[:split, :, :D], cache[:split, :, D:]
+                if tail is None:
+                    core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
+                                              out=core_dst, return_lse=False, q_prescaled=True, score_bound=bound_core)
+                else:
+                    core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
+                                              k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, out=core_dst,
+                                              return_lse=False, q_prescaled=True, score_bound=bound_core)
+                persisted = n_keep
+            finally:
+                if offloaded is not None:  # the persisted rows go back to the host behind the attention launch
+                    offloaded.release(start, persisted)
         if fused is not None:
             if self._cross_attention_fused(qx_raw, key_value_states, meta_args.cross_attn_params, cross_dst) is None:
                 self.cross_attention(mixed_qqkv, key_value_states, meta_args.cross_attn_params, get_xqkv, out=cross_dst)

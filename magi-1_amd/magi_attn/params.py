@@ -51,8 +51,9 @@ class InferenceParams:
     """Run-time state of one generation: the per-layer KV cache (dataclass.py:62-71).
 
     key_value_memory_dict[layer_number] is a [max_sequence_length * max_batch_size, Hkv, 2*D]
-    tensor, K in [..., :D] and V in [..., D:].  On MI355X it always lives in HBM (288 GB holds
-    every layer of the 24B model at 720p), so there is no host-offload variant."""
+    tensor, K in [..., :D] and V in [..., D:].  On MI355X it normally lives in HBM (288 GB hold
+    every layer of the 24B model at 720p); a KVCacheArena(kv_offload=True) puts OffloadedKVCache
+    objects here instead (pinned host memory behind device staging buffers)."""
 
     def __init__(self, max_batch_size: int, max_sequence_length: int):
         self.max_sequence_length = max_sequence_length
@@ -74,7 +75,7 @@ class InferenceParams:
             raise ValueError("batch_idx must name every batch row once")
         for layer_number, cache in self.key_value_memory_dict.items():
             if not isinstance(cache, torch.Tensor):
-                raise TypeError("swap_key_value_dict works on tensor caches (not on an Fp8KVCache)")
+                raise TypeError("swap_key_value_dict works on tensor caches (not on an Fp8KVCache or an offloaded cache)")
             rows = cache.view(self.max_sequence_length, self.max_batch_size, *cache.shape[1:])
             self.key_value_memory_dict[layer_number] = rows[:, idx.to(cache.device)].reshape(cache.shape)
 

@@ -231,7 +231,11 @@ def test_kv_cache_arena_views_accounting_and_errors():
     with pytest.raises(MemoryError):
         KVCacheArena(48, 259200, 8, device="cpu", memory_budget_bytes=1 << 30)
     with pytest.raises(ValueError):
-        KVCacheArena(1, 8, 1, device="cpu", kv_offload=True)
+        KVCacheArena(1, 8, 1, device="cpu", kv_offload=True)   # the staging buffers need a GPU
+    with pytest.raises(ValueError):
+        KVCacheArena(1, 8, 1, device="cuda", kv_offload=True, max_batch_size=2)
+    with pytest.raises(MemoryError):                              # with kv_offload the budget counts the staging ring
+        KVCacheArena(48, 259200, 8, device="cuda", kv_offload=True, memory_budget_bytes=1 << 30)
 
 
 def test_projection_weights_share_one_buffer():

@@ -536,6 +536,74 @@ def test_layer_with_arena_backed_cache(dev):
     assert torch.isnan(arena.layer(2)).all() and torch.isnan(arena.layer(4)).all()  # other layers untouched
 
 
+@pytest.mark.parametrize("staging_buffers", [1, 2, 3])
+def test_layers_with_offloaded_caches_match_resident_ones(dev, staging_buffers):
+    """kv_offload as an option (dit_module.py:803-811, 915): three layers whose caches live in pinned host memory behind
+    a ring of 1, 2 or 3 device staging buffers, run through a schedule that appends, re-reads without persisting
+    (update_kv_cache False: side buffer), drops the last chunk (distill) and then starts a second generation on the
+    same arena with different inputs (a copy made ahead for the next layer must not survive a rewrite of the host
+    rows).  Every output and every persisted cache row is bit-identical to the same schedule on a resident arena."""
+    from magi_attn.cache import KVCacheArena, OffloadedKVCache
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+    hidden, Hq, Hkv, D = 256, 6, 2, 128
+    fr, H, W = 1, 4, 4
+    L = fr * H * W
+    n_chunks = 6
+    layers = []
+    for i in range(3):
+        torch.manual_seed(40 + i)
+        layer = MOD.FullyParallelAttention(hidden, Hq, Hkv, layer_number=i, device=dev)
+        with torch.no_grad():
+            for prm in layer.parameters():
+                prm.copy_(torch.randn_like(prm.float()) * (0.1 if prm.dim() == 1 else hidden ** -0.5))
+            layer.linear_qkv.layer_norm.weight.add_(1.0)
+        layers.append(layer)
+    rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
+    # (slice_point, denoising chunks, update_kv_cache, distill_nearly_clean_chunk)
+    schedule = [(0, 2, True, False), (2, 2, False, False), (2, 2, True, True), (3, 3, True, False),
+                (0, 2, True, False), (2, 3, True, False)]          # the last two: a new generation on the same arena
+    results = []
+    for offload in (False, True):
+        arena = KVCacheArena(3, n_chunks * L, Hkv, device=dev, kv_offload=offload, staging_buffers=staging_buffers)
+        ip = P.InferenceParams(1, n_chunks * L)
+        arena.attach(ip)
+        if offload:
+            assert all(isinstance(ip.key_value_memory_dict[i], OffloadedKVCache) for i in range(3))
+            assert arena.host.is_pinned() and len(arena.stages) == min(3, staging_buffers)
+        g = torch.Generator().manual_seed(9)
+        outs, rows = [], []
+        for sp, dn, update, distill in schedule:
+            ip.update_kv_cache = update
+            S = dn * L
+            hs = torch.randn(S, 1, hidden, generator=g).bfloat16().to(dev)
+            y = (torch.randn(dn * 8, hidden, generator=g) * 0.5).bfloat16().to(dev)
+            meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=sp,
+                                   denoising_range_num=dn, range_num=sp + dn, extract_prefix_video_feature=False,
+                                   fwd_extra_1st_chunk=True, distill_nearly_clean_chunk=distill, clip_token_nums=L,
+                                   enable_cuda_graph=False,
+                                   core_attn_params=P.build_core_attn_params(R.q_ranges_from_chunks(dn, L).to(dev),
+                                                                             R.generate_default_kvrange(sp, dn, L).to(dev), L),
+                                   cross_attn_params=P.build_cross_attn_params(torch.ones(dn, 1, 1, 8).to(dev), L, 8))
+            rope = rope_mod.get_embed_for_forward(dn * fr, H, W, sp, dn)
+            x = hs
+            with torch.no_grad():
+                for layer in layers:       # each layer's self-attention output feeds the next (hidden = Hq * D / 3)
+                    core, cross = layer(x, y, ip, rope, meta)
+                    outs.append((core.clone(), cross.clone()))
+                    x = (core.view(S, 1, 3, hidden).float().mean(2) + hs.float()).bfloat16()
+            arena.synchronize()
+            kept = (sp + (dn - 1 if distill else dn)) * L if update else None
+            if kept is not None:
+                src = arena.host if offload else arena.buffer
+                rows.append(src[:, sp * L:kept].clone().cpu())
+        results.append((outs, rows))
+    for (c0, x0), (c1, x1) in zip(*[r[0] for r in results]):
+        assert torch.equal(c0, c1) and torch.equal(x0, x1)
+    assert len(results[0][1]) == len(results[1][1]) == 5
+    for r0, r1 in zip(results[0][1], results[1][1]):
+        assert torch.equal(r0, r1)
+
+
 @pytest.mark.parametrize("fast_exp2", [True, False])
 def test_layer_with_fp8_self_attention_and_fp8_cache(dev, fast_exp2):
     """attention_dtype="fp8": same schedule as above through two layers with identical weights, one bf16 and one

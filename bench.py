@@ -486,9 +486,9 @@ def mfma_ceiling_leg(dev):
 
 def secondary_legs(inp, dev, steps):
     """Core-attention launches the headline does not time, kernel only, a few steps each: the online-softmax kernel a
-    caller without a score bound gets (unscaled q), the bounded kernel fed with unscaled q and a bound (what the
-    reference-shaped callables select: it scales q while loading it), the shipped sliding window on the same layer,
-    and the 480p 4.5B-style layer."""
+    caller gets who neither states a score bound nor lets the library measure one (unscaled q), the bounded kernel
+    fed with unscaled q and a bound (it scales q while loading it), the reference's unchanged call with the bound
+    measured by the library, the shipped sliding window on the same layer, and the 480p 4.5B-style layer."""
     import magi_attn as M
     from magi_attn import ranges as R
 
@@ -512,6 +512,13 @@ def secondary_legs(inp, dev, steps):
     ms = timed(lambda: M.range_attention(q_unscaled, k, v, inp["q_ranges"], inp["k_ranges"], L, out=inp["out"],
                                          return_lse=False, score_bound=SCORE_BOUND), steps)
     res["bounded_unscaled_q_scale_on_load"] = entry(ms, core_fl, "attn_fwd_bf16_x16_kernel (q scaled while loaded)")
+    # the reference's own call, nothing added: unscaled q, no bound.  The library measures max|q| max|k| in two passes and
+    # both kernels are launched behind them (MAGI_ATTN_AUTO_BOUND); the time is that of all five launches.
+    assert M.functional._measuring_a_bound_pays(q_unscaled, k, dn, L, (sp + dn) * L)
+    ms = timed(lambda: M.range_attention(q_unscaled, k, v, inp["q_ranges"], inp["k_ranges"], L, (sp + dn) * L, out=inp["out"],
+                                         return_lse=False, auto_bound=True), steps)
+    res["reference_call_unchanged_measured_bound"] = entry(
+        ms, core_fl, "row_norm_max_kernel x 2 + attn_fwd_bf16_x16_kernel (selected on the device) + attn_fwd_bf16_kernel (returns at once)")
     del q_unscaled
     # the bounded kernel's 32x32x16-MFMA form (MAGI_ATTN_BOUNDED_MFMA32) on the headline's inputs: same box, same run
     ms = timed(lambda: M.range_attention(inp["q"], k, v, inp["q_ranges"], inp["k_ranges"], L, out=inp["out"],

@@ -51,11 +51,13 @@ int compute_units() {
   return cached[dev];
 }
 
+int attn_fwd_impl(const magi_attn_args* p, void* stream, float* workspace);
+
 }  // namespace
 
 extern "C" {
 
-int magi_version(void) { return 102; }
+int magi_version(void) { return 103; }
 
 uint64_t magi_launch_count(void) { return g_launches.load(std::memory_order_relaxed); }
 
@@ -64,6 +66,14 @@ const char* magi_last_error(void) { return g_err; }
 int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   if (!p) return fail(MAGI_EINVAL, "magi_attn_fwd: args is NULL");
   MAGI_CHECK_LAYOUT("magi_attn_fwd", p);
+  return attn_fwd_impl(p, stream, p->workspace);
+}
+
+}  // extern "C"
+
+namespace {
+
+int attn_fwd_impl(const magi_attn_args* p, void* stream, float* workspace) {
   if (p->D != 128) return fail(MAGI_ENOSYS, "magi_attn_fwd: head_dim %d not implemented (128 only)", p->D);
   if (p->dtype != MAGI_DTYPE_BF16 && p->dtype != MAGI_DTYPE_FP8_E4M3)
     return fail(MAGI_EINVAL, "magi_attn_fwd: unknown dtype %d", p->dtype);
@@ -116,6 +126,15 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   }
   if (p->score_bound > 0.f && p->dtype != MAGI_DTYPE_BF16)
     return fail(MAGI_EINVAL, "magi_attn_fwd: score_bound is a promise about bf16 inputs");
+  const bool auto_bound = (p->flags & MAGI_ATTN_AUTO_BOUND) != 0;
+  if (auto_bound) {
+    if (p->dtype != MAGI_DTYPE_BF16 || p->score_bound > 0.f || q_norm || p->q_tile_rows != 0 ||
+        (p->flags & MAGI_ATTN_BOUNDED_MFMA32))
+      return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_AUTO_BOUND goes with bf16 and without score_bound, q_norm, "
+                               "q_tile_rows and MAGI_ATTN_BOUNDED_MFMA32 (it measures the bound and picks the kernel itself)");
+    if (!workspace || !aligned16(workspace))
+      return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_AUTO_BOUND needs a 16-byte workspace on the device, 16-byte aligned");
+  }
   if (p->out_group_heads < 0 || (p->out_group_heads > 0 && (p->Hq % p->out_group_heads || p->o_stride_g % 8)))
     return fail(MAGI_EINVAL, "magi_attn_fwd: out_group_heads must divide Hq and o_stride_g keep rows 16-byte aligned");
   int k_split = p->total_k;
@@ -177,33 +196,12 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   //    every K / V tile fetched once for three times as many rows and one barrier per tile) pay on grids of many
   //    rounds with long key ranges (measured: +3 % at 43 rounds, +1 % at 9.4, -3 % at 5.3); small grids and short
   //    key ranges (cross attention) keep 128 rows (4 waves, three workgroups per CU).
-  a.block_m = 128;
   if (p->dtype == MAGI_DTYPE_FP8_E4M3 && p->q_tile_rows != 0 && p->q_tile_rows != 128)
     return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (fp8: 128)", p->q_tile_rows);
-  const bool bounded = p->dtype == MAGI_DTYPE_BF16 && p->score_bound > 0.f && p->score_bound <= MAGI_SCORE_BOUND_MAX;
-  // a bound stated for unscaled q (what the reference's callers pass): the kernel applies the softmax scale while it
-  // loads q, after which the scores are exp2 exponents as with MAGI_ATTN_Q_PRESCALED
-  const bool scale_q = bounded && !q_norm && !(p->flags & MAGI_ATTN_Q_PRESCALED);
+  const bool promised = p->dtype == MAGI_DTYPE_BF16 && p->score_bound > 0.f && p->score_bound <= MAGI_SCORE_BOUND_MAX;
   const bool mfma32 = (p->flags & MAGI_ATTN_BOUNDED_MFMA32) != 0;
-  if (mfma32 && !(bounded && (p->flags & MAGI_ATTN_Q_PRESCALED)))
+  if (mfma32 && !(promised && (p->flags & MAGI_ATTN_Q_PRESCALED)))
     return fail(MAGI_EINVAL, "magi_attn_fwd: MAGI_ATTN_BOUNDED_MFMA32 goes with bf16, MAGI_ATTN_Q_PRESCALED and a score_bound in force");
-  if (p->dtype == MAGI_DTYPE_BF16) {
-    const double wg384 = (double)p->Hq * p->n_ranges * ((p->max_seqlen_q + 383) / 384);
-    const bool long_keys = p->max_seqlen_k == 0 || p->max_seqlen_k >= 4096;  // (0 = not stated)
-    if (bounded)
-      a.block_m = 256;  // (512-row workgroups fetch half the tiles and measure 1 % slower: their two waves per SIMD march in step)
-    else if (wg384 >= 9.0 * compute_units() && long_keys)
-      a.block_m = 384;
-    if (p->q_tile_rows != 0) {
-      const int r = p->q_tile_rows;
-      if ((q_norm || scale_q) && r != 256)
-        return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (with q_norm, or a score bound on unscaled q: 256)", r);
-      if (bounded ? (r != 256 && r != 512) : (r != 128 && r != 384))
-        return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (bf16: 128 or 384; with a score bound: 256 or 512)", r);
-      a.block_m = r;
-    }
-  }
-  a.tiles_per_range = (p->max_seqlen_q + a.block_m - 1) / a.block_m;
   a.Hq = p->Hq;
   a.Hkv = p->Hkv;
   a.G = p->Hq / p->Hkv;
@@ -214,30 +212,79 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
     a.k2_scale_delta = (p->k2_scale - p->k_scale) - (long)a.scale_split_chunk * p->Hkv;
     a.v2_scale_delta = (p->v2_scale - p->v_scale) - (long)a.scale_split_chunk * p->Hkv;
   }
-  a.flags = p->flags | (bounded ? magi::ATTN_BOUNDED : 0) | (scale_q ? magi::ATTN_SCALE_Q : 0);
-  const double total = (double)p->Hq * p->n_ranges * a.tiles_per_range;
-  if (total > 2.0e9) return fail(MAGI_EINVAL, "magi_attn_fwd: grid too large (%.3g workgroups)", total);
-  a.total_wgs = (unsigned)total;
-  a.per_xcd = (a.total_wgs + 7u) / 8u;
   const float scale = p->softmax_scale > 0.f ? p->softmax_scale : 1.0f / std::sqrt((float)p->D);
   a.scale_log2 = scale * 1.4426950408889634f;
   if (p->dtype == MAGI_DTYPE_BF16 && (p->flags & MAGI_ATTN_Q_PRESCALED)) a.scale_log2 = 1.f;  // q . k is the exp2 exponent
   // (with q_norm, or a score bound on unscaled q, the kernel multiplies q by scale_log2 itself while loading it, after
   // which the same holds)
 
-  hipError_t e;
-  if (p->dtype != MAGI_DTYPE_BF16)
-    e = magi::launch_attn_fwd_fp8(a, static_cast<hipStream_t>(stream));
-  else if (bounded && a.block_m == 256 && !mfma32)
-    e = magi::launch_attn_fwd_bf16_x16(a, static_cast<hipStream_t>(stream));
-  else if (bounded)
-    e = magi::launch_attn_fwd_bf16_w64(a, static_cast<hipStream_t>(stream));
-  else
-    e = magi::launch_attn_fwd_bf16(a, static_cast<hipStream_t>(stream));
-  if (e != hipSuccess) return hip_fail(e, "magi_attn_fwd launch");
-  g_launches.fetch_add(1, std::memory_order_relaxed);
-  return MAGI_OK;
+  // One launch of `a` as the bounded-score kernel (bounded) or as the kernel without a promise about the scores.
+  auto launch = [&](bool bounded) -> int {
+    // a bound stated for unscaled q (what the reference's callers pass): the kernel applies the softmax scale while
+    // it loads q, after which the scores are exp2 exponents as with MAGI_ATTN_Q_PRESCALED
+    const bool scale_q = bounded && !q_norm && !(p->flags & MAGI_ATTN_Q_PRESCALED);
+    a.block_m = 128;
+    if (p->dtype == MAGI_DTYPE_BF16) {
+      const double wg384 = (double)p->Hq * p->n_ranges * ((p->max_seqlen_q + 383) / 384);
+      const bool long_keys = p->max_seqlen_k == 0 || p->max_seqlen_k >= 4096;  // (0 = not stated)
+      if (bounded)
+        a.block_m = 256;  // (512-row workgroups fetch half the tiles and measure 1 % slower: their two waves per SIMD march in step)
+      else if (wg384 >= 9.0 * compute_units() && long_keys)
+        a.block_m = 384;
+      if (p->q_tile_rows != 0) {
+        const int r = p->q_tile_rows;
+        if ((q_norm || scale_q) && r != 256)
+          return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (with q_norm, or a score bound on unscaled q: 256)", r);
+        if (bounded ? (r != 256 && r != 512) : (r != 128 && r != 384))
+          return fail(MAGI_EINVAL, "magi_attn_fwd: q_tile_rows %d (bf16: 128 or 384; with a score bound: 256 or 512)", r);
+        a.block_m = r;
+      }
+    }
+    a.tiles_per_range = (p->max_seqlen_q + a.block_m - 1) / a.block_m;
+    a.flags = p->flags | (bounded ? magi::ATTN_BOUNDED : 0) | (scale_q ? magi::ATTN_SCALE_Q : 0);
+    const double total = (double)p->Hq * p->n_ranges * a.tiles_per_range;
+    if (total > 2.0e9) return fail(MAGI_EINVAL, "magi_attn_fwd: grid too large (%.3g workgroups)", total);
+    a.total_wgs = (unsigned)total;
+    a.per_xcd = (a.total_wgs + 7u) / 8u;
+    hipError_t e;
+    if (p->dtype != MAGI_DTYPE_BF16)
+      e = magi::launch_attn_fwd_fp8(a, static_cast<hipStream_t>(stream));
+    else if (bounded && a.block_m == 256 && !mfma32)
+      e = magi::launch_attn_fwd_bf16_x16(a, static_cast<hipStream_t>(stream));
+    else if (bounded)
+      e = magi::launch_attn_fwd_bf16_w64(a, static_cast<hipStream_t>(stream));
+    else
+      e = magi::launch_attn_fwd_bf16(a, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return hip_fail(e, "magi_attn_fwd launch");
+    g_launches.fetch_add(1, std::memory_order_relaxed);
+    return MAGI_OK;
+  };
+
+  if (!auto_bound) return launch(promised);
+
+  // No promise about the scores: measure one.  Two streaming passes leave the largest squared length of a q row and
+  // of a k row in the workspace (|q . k| <= |q| |k|); both attention kernels are launched behind them, each tests
+  // the bound on the device and only the one it selects runs (the other returns at once).  No host synchronisation.
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  unsigned* ws = reinterpret_cast<unsigned*>(workspace);
+  hipError_t e = magi::launch_gate_init(ws, st);
+  if (e == hipSuccess) e = magi::launch_row_norm_max(a.q, a.qs_t, a.qs_h, p->total_q, p->Hq, ws, st);
+  if (e == hipSuccess && k_split > 0) e = magi::launch_row_norm_max(a.k, a.ks_t, a.ks_h, k_split, p->Hkv, ws + 1, st);
+  if (e == hipSuccess && p->total_k > k_split)
+    e = magi::launch_row_norm_max(a.k2, a.ks_t, a.ks_h, p->total_k - k_split, p->Hkv, ws + 1, st);
+  if (e != hipSuccess) return hip_fail(e, "magi_attn_fwd bound measurement");
+  g_launches.fetch_add(2 + (k_split > 0) + (p->total_k > k_split), std::memory_order_relaxed);
+  a.gate = workspace;
+  a.gate_want = 1;
+  int rc = launch(true);
+  if (rc != MAGI_OK) return rc;
+  a.gate_want = 0;
+  return launch(false);
 }
+
+}  // namespace
+
+extern "C" {
 
 int magi_qk_prologue(const magi_prologue_args* p, void* stream) {
   if (!p) return fail(MAGI_EINVAL, "magi_qk_prologue: args is NULL");

@@ -66,6 +66,16 @@ __device__ __forceinline__ float pair_sum(unsigned pk, float acc) {
   return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, pk), one, acc, false);
 }
 
+// A launch behind a measured score bound: true when this kernel is not the one the bound selects (every thread of
+// the grid sees the same two values, so the whole launch returns).  NaN lengths fail the comparison and select the
+// online-softmax kernel.
+__device__ __forceinline__ bool gate_closed(const AttnKernArgs& a) {
+  if (!a.gate) return false;
+  const float b = __builtin_sqrtf(a.gate[0] * a.gate[1]) * a.scale_log2 * 1.01f;
+  const bool fits = b <= 64.0f;  // MAGI_SCORE_BOUND_MAX
+  return fits != (a.gate_want != 0);
+}
+
 // What one workgroup works on: q rows [q0, min(q0 + BM, qe)) of head h against keys [ks, ke) of kv head kvh.
 struct WorkItem {
   int h, kvh;

@@ -69,6 +69,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   static_assert(DB != VSINGLE, "one of the two tile loops");
   __shared__ int s_sel;
 
+  if (gate_closed(a)) return;
   const int tid = threadIdx.x;
   // ---- which piece of work is this workgroup? ----
   const WorkItem wi = locate_work(a, BM, tid, &s_sel);

@@ -70,6 +70,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   __shared__ __attribute__((aligned(1024))) unsigned char sV1[TILE_BYTES];
   __shared__ int s_sel;
 
+  if (gate_closed(a)) return;
   const int tid = threadIdx.x;
   const WorkItem wi = locate_work(a, BM, tid, &s_sel);
   if (!wi.valid) return;

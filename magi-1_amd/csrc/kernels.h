@@ -38,6 +38,12 @@ struct AttnKernArgs {
   float scale_log2;  // softmax_scale * log2(e)
   float q_norm_eps;
   int q_norm_kind;  // MAGI_NORM_LAYERNORM_1P / MAGI_NORM_RMSNORM_1P
+  // Measured score bound (MAGI_ATTN_AUTO_BOUND): gate[0] / gate[1] = the largest squared length of a q row / a k row
+  // as launch_row_norm_max left them.  A kernel that is handed a gate first tests whether
+  // sqrt(gate[0] gate[1]) * scale_log2 * 1.01 <= MAGI_SCORE_BOUND_MAX and runs only if the answer equals
+  // gate_want (the bounded-score kernel: 1, the online-softmax kernel launched behind it: 0).  NULL: no test.
+  const float* gate;
+  int gate_want;
 };
 
 
@@ -50,6 +56,12 @@ hipError_t launch_attn_fwd_bf16(const AttnKernArgs& a, hipStream_t stream);
 hipError_t launch_attn_fwd_bf16_w64(const AttnKernArgs& a, hipStream_t stream);
 hipError_t launch_attn_fwd_bf16_x16(const AttnKernArgs& a, hipStream_t stream);
 hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream);
+// ws[0..3] = 0 (a kernel, not a memset: the call may be under graph capture)
+hipError_t launch_gate_init(unsigned* ws, hipStream_t stream);
+// *out_bits = max(*out_bits, bit pattern of the largest sum of squares over a [T, H, 128] bf16 tensor's rows);
+// strides in BYTES.  Bit patterns of non-negative floats order like the floats, and a NaN row ends up on top.
+hipError_t launch_row_norm_max(const char* x, long stride_t, long stride_h, int T, int H, unsigned* out_bits,
+                               hipStream_t stream);
 
 struct PrologueKernArgs {
   const char* q_raw;

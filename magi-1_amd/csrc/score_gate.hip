@@ -1,0 +1,64 @@
+// Measured score bound for callers that state none (MAGI_ATTN_AUTO_BOUND): one streaming pass over q and one over k
+// leave the largest squared row length of each in two words of a caller-provided workspace.  By Cauchy-Schwarz
+// |q . k| <= |q| |k| for every pair, so the attention kernels launched behind these passes can decide ON THE DEVICE,
+// with no host synchronisation, whether the bounded-score kernel applies (it does for QK-normed attention at ordinary
+// gains) or the online-softmax kernel has to run.  HBM bound, 256 bytes per (token, head) row.
+#include <hip/hip_runtime.h>
+
+#include "kernels.h"
+
+namespace magi {
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+__global__ void gate_init_kernel(unsigned* ws) {
+  if (threadIdx.x < 4) ws[threadIdx.x] = 0u;
+}
+
+// 16 lanes per row of 128 bf16 values (16 bytes each); a workgroup of 256 threads walks 16 rows at a time with a
+// grid stride.  The maximum is taken on bit patterns: sums of squares are non-negative, so their patterns order like
+// their values, infinity lies above every finite sum and a NaN above infinity (whatever its sign bit): a tensor with
+// a NaN row reports a NaN length, which no bound test passes.
+__global__ __launch_bounds__(256) void row_norm_max_kernel(const char* __restrict__ x, long stride_t, long stride_h,
+                                                           int T, int H, unsigned* __restrict__ out_bits) {
+  const int sub = threadIdx.x & 15;
+  const long rows = (long)T * H;
+  const long step = (long)gridDim.x * 16;
+  unsigned best = 0u;
+  for (long r = (long)blockIdx.x * 16 + (threadIdx.x >> 4); r < rows; r += step) {
+    const long t = r / H;
+    const int h = (int)(r - t * H);
+    const bf16x8 v = *(const bf16x8*)(x + t * stride_t + (long)h * stride_h + sub * 16);
+    float s = 0.f;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) s += (float)v[e] * (float)v[e];
+    s += __shfl_xor(s, 1);
+    s += __shfl_xor(s, 2);
+    s += __shfl_xor(s, 4);
+    s += __shfl_xor(s, 8);
+    best = max(best, __float_as_uint(s));
+  }
+  best = max(best, (unsigned)__shfl_xor((int)best, 16));
+  best = max(best, (unsigned)__shfl_xor((int)best, 32));
+  if ((threadIdx.x & 63) == 0 && best != 0u) atomicMax(out_bits, best);
+}
+
+}  // namespace
+
+hipError_t launch_gate_init(unsigned* ws, hipStream_t stream) {
+  hipLaunchKernelGGL(gate_init_kernel, dim3(1), dim3(64), 0, stream, ws);
+  return hipGetLastError();
+}
+
+hipError_t launch_row_norm_max(const char* x, long stride_t, long stride_h, int T, int H, unsigned* out_bits,
+                               hipStream_t stream) {
+  const long rows = (long)T * H;
+  if (rows <= 0) return hipSuccess;
+  const long want = (rows + 15) / 16;
+  const unsigned blocks = (unsigned)(want < 4096 ? want : 4096);
+  hipLaunchKernelGGL(row_norm_max_kernel, dim3(blocks), dim3(256), 0, stream, x, stride_t, stride_h, T, H, out_bits);
+  return hipGetLastError();
+}
+
+}  // namespace magi

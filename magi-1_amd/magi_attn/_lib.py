@@ -22,6 +22,7 @@ MAGI_ATTN_FP8_POW2_PRESCALED = 1
 MAGI_ATTN_Q_PRESCALED = 2
 MAGI_ATTN_FP8_FAST_EXP2 = 4
 MAGI_ATTN_BOUNDED_MFMA32 = 8
+MAGI_ATTN_AUTO_BOUND = 16
 MAGI_SCORE_BOUND_MAX = 64.0
 
 
@@ -59,6 +60,7 @@ class AttnArgs(_SizedStructure):
         ("q_tile_rows", C.c_int32),
         ("q_norm_gamma", C.c_void_p), ("q_norm_beta", C.c_void_p), ("q_norm_eps", C.c_float), ("q_norm_kind", C.c_int32),
         ("k2_scale", C.c_void_p), ("v2_scale", C.c_void_p),
+        ("workspace", C.c_void_p),
     ]
 
 
@@ -103,9 +105,10 @@ class QuantizeArgs(_SizedStructure):
     ]
 
 
-ABI_VERSION = 102  # magi_version() of the library these mirrors were written for
+ABI_VERSION = 103  # magi_version() of the library these mirrors were written for
 
-EXPORTS = ("magi_version", "magi_last_error", "magi_launch_count", "magi_attn_fwd", "magi_qk_prologue", "magi_head_norm",
+EXPORTS = ("magi_version", "magi_last_error", "magi_launch_count", "magi_attn_fwd",
+           "magi_qk_prologue", "magi_head_norm",
            "magi_apply_rotary", "magi_quantize_fp8", "magi_quantize_fp8_split", "magi_layer_norm", "magi_qkv_proj_prologue", "magi_div_clamp_to_e4m3")
 
 _lib = None

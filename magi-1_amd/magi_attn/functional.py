@@ -74,6 +74,7 @@ def range_attention(
     score_bound: float = 0.0,
     q_tile_rows: int = 0,
     bounded_mfma32: bool = False,
+    auto_bound: bool = False,
     q_norm: Optional[tuple] = None,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = True,
@@ -97,6 +98,9 @@ def range_attention(
     it loads q.
     q_tile_rows: force a workgroup shape (0 = the library's choice); see magi_attn_args.q_tile_rows.
     bounded_mfma32 (with q_prescaled and score_bound): the 32x32x16 form of the bounded kernel, MAGI_ATTN_BOUNDED_MFMA32.
+    auto_bound (bf16, instead of score_bound): the library measures max|q| and max|k| in two streaming passes and
+    picks the bounded-score kernel on the device when their product allows it, MAGI_ATTN_AUTO_BOUND (its 16-byte
+    workspace is a fresh tensor).
     q_norm: (gamma, beta or None, eps[, norm_kind]): q is the raw projection, normalised per (token, head) row inside
     the kernel (fp32, zero-centred gamma) and scaled by softmax_scale * log2(e); needs score_bound.
     """
@@ -173,7 +177,12 @@ def range_attention(
     a.scale_chunk_tokens = int(scale_chunk_tokens)
     a.softmax_scale = 0.0 if softmax_scale is None else float(softmax_scale)
     a.flags = ((L.MAGI_ATTN_FP8_POW2_PRESCALED if fp8_pow2_prescaled else 0) | (L.MAGI_ATTN_Q_PRESCALED if q_prescaled else 0)
-               | (L.MAGI_ATTN_FP8_FAST_EXP2 if fp8_fast_exp2 else 0) | (L.MAGI_ATTN_BOUNDED_MFMA32 if bounded_mfma32 else 0))
+               | (L.MAGI_ATTN_FP8_FAST_EXP2 if fp8_fast_exp2 else 0) | (L.MAGI_ATTN_BOUNDED_MFMA32 if bounded_mfma32 else 0)
+               | (L.MAGI_ATTN_AUTO_BOUND if auto_bound else 0))
+    workspace = None
+    if auto_bound:
+        workspace = torch.empty(4, dtype=torch.float32, device=q.device)  # (alive until the launches are enqueued)
+        a.workspace = _ptr(workspace)
     a.score_bound = float(score_bound)
     a.q_tile_rows = int(q_tile_rows)
     keep = None
@@ -198,23 +207,44 @@ def qk_norm_score_bound(q_norm_bound: float, k_norm_bound: float, head_dim: int 
     return 1.01 * scale * math.log2(math.e) * q_norm_bound * k_norm_bound
 
 
+def _measuring_a_bound_pays(q, k, n_ranges: int, max_seqlen_q: int, max_seqlen_k: int) -> bool:
+    """A bf16 call without a score_bound: are the two passes of MAGI_ATTN_AUTO_BOUND (one over q, one over k) small
+    beside what the bounded-score kernel saves?  Decided from sizes the host knows, generously on the side of the
+    plain online-softmax launch: the saving is put at 12 % of the attention time, the passes at twice their HBM time
+    plus three launches."""
+    if q.dtype != torch.bfloat16 or q.dim() != 3 or q.shape[-1] != 128:
+        return False
+    Tq, Hq, D = q.shape
+    keys = max_seqlen_k if max_seqlen_k > 0 else k.shape[0]
+    attention_s = 4.0 * D * Hq * min(Tq, max(n_ranges, 0) * max_seqlen_q) * keys / 1.2e15
+    passes_s = (Tq * Hq + k.shape[0] * k.shape[1]) * 2 * D / 4e12 + 3e-5
+    return 0.12 * attention_s > 2 * passes_s
+
+
 def flex_flash_attn_func(q, k, v, q_ranges, k_ranges, max_seqlen_q, max_seqlen_k, softmax_scale=None,
-                         deterministic=False, disable_fwd_atomic_reduction=True, score_bound: float = 0.0, **_unused):
+                         deterministic=False, disable_fwd_atomic_reduction=True, score_bound: float = 0.0,
+                         auto_bound: Optional[bool] = None, **_unused):
     """(out [Tq,Hq,D], lse [Hq,Tq]) for disjoint q ranges.  The forward has one writer per output
     row, so it is deterministic and needs no atomic reduction whatever the two flags say.
 
     score_bound (no counterpart in the reference's call, optional): the caller's promise that
     |q . k| * softmax_scale * log2(e) <= score_bound for every pair, with q unscaled as the reference passes it
     (qk_norm_score_bound derives it from the norm parameters).  Up to MAGI_SCORE_BOUND_MAX it selects the kernel
-    without a running maximum, which applies the scale while it loads q."""
+    without a running maximum, which applies the scale while it loads q.
+
+    auto_bound: without a score_bound the library can measure one (range_attention's auto_bound).  None (default):
+    it does where the two passes over q and k are small beside the attention itself, which is how the reference's
+    own call, unchanged, reaches the bounded-score kernel on its QK-normed q and k."""
+    if auto_bound is None:
+        auto_bound = score_bound == 0.0 and _measuring_a_bound_pays(q, k, q_ranges.shape[0], max_seqlen_q, max_seqlen_k)
     return range_attention(q, k, v, q_ranges, k_ranges, max_seqlen_q, max_seqlen_k, softmax_scale,
-                           score_bound=score_bound)
+                           score_bound=score_bound, auto_bound=bool(auto_bound) and score_bound == 0.0)
 
 
 def flash_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, deterministic=False,
-                    score_bound: float = 0.0, **_unused):
+                    score_bound: float = 0.0, auto_bound: Optional[bool] = None, **_unused):
     """q [B,Sq,Hq,D], k/v [B,Sk,Hkv,D] -> [B,Sq,Hq,D]; non-causal, no dropout (what the reference uses).
-    score_bound: as in flex_flash_attn_func."""
+    score_bound, auto_bound: as in flex_flash_attn_func."""
     if dropout_p != 0.0 or causal:
         raise NotImplementedError("dropout / causal are not part of the MAGI-1 attention path")
     B, Sq, Hq, D = q.shape
@@ -224,19 +254,26 @@ def flash_attn_func(q, k, v, dropout_p=0.0, softmax_scale=None, causal=False, de
     v3 = v.reshape(B * Sk, v.shape[2], D)
     cu_q = torch.arange(0, (B + 1) * Sq, Sq, dtype=torch.int32, device=q.device)
     cu_k = torch.arange(0, (B + 1) * Sk, Sk, dtype=torch.int32, device=q.device)
+    if auto_bound is None:
+        auto_bound = score_bound == 0.0 and _measuring_a_bound_pays(q3, k3, B, Sq, Sk)
     out, _ = range_attention(q3, k3, v3, cu_q, cu_k, Sq, Sk, softmax_scale, ranges_mode=L.MAGI_RANGES_CU,
-                             return_lse=False, zero_init=False, score_bound=score_bound)
+                             return_lse=False, zero_init=False, score_bound=score_bound,
+                             auto_bound=bool(auto_bound) and score_bound == 0.0)
     return out.view(B, Sq, Hq, D)
 
 
 def flash_attn_varlen_func(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, dropout_p=0.0,
-                           softmax_scale=None, causal=False, deterministic=False, score_bound: float = 0.0, **_unused):
+                           softmax_scale=None, causal=False, deterministic=False, score_bound: float = 0.0,
+                           auto_bound: Optional[bool] = None, **_unused):
     """Packed varlen attention; segment s pairs q[cu_q[s]:cu_q[s+1]] with k[cu_k[s]:cu_k[s+1]].
-    A segment without keys yields zero rows.  score_bound: as in flex_flash_attn_func."""
+    A segment without keys yields zero rows.  score_bound, auto_bound: as in flex_flash_attn_func."""
     if dropout_p != 0.0 or causal:
         raise NotImplementedError("dropout / causal are not part of the MAGI-1 attention path")
+    if auto_bound is None:
+        auto_bound = score_bound == 0.0 and _measuring_a_bound_pays(q, k, cu_seqlens_q.numel() - 1, max_seqlen_q, max_seqlen_k)
     out, _ = range_attention(q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale,
-                             ranges_mode=L.MAGI_RANGES_CU, return_lse=False, zero_init=True, score_bound=score_bound)
+                             ranges_mode=L.MAGI_RANGES_CU, return_lse=False, zero_init=True, score_bound=score_bound,
+                             auto_bound=bool(auto_bound) and score_bound == 0.0)
     return out
 
 

@@ -206,6 +206,17 @@ typedef struct magi_attn_args {
 int magi_attn_fwd(const magi_attn_args* args, void* stream);
 
 /*
+ * magi_attn_fwd for callers that cannot hand over a workspace and must not allocate one (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc): args->workspace is ignored, and the scratch
+ * memory of MAGI_ATTN_AUTO_BOUND is a 256-byte array that lives in the library's device image, one copy per GPU, held
+ * until the process ends.  Its need does not grow with the problem (four words), so no size is refused for it.
+ * Calls that overlap on one GPU (two streams, two threads) share the array and race: issue them on one stream, or
+ * give the others a workspace through magi_attn_fwd.  Without MAGI_ATTN_AUTO_BOUND it is magi_attn_fwd.  Allocates
+ * nothing, like every entry point of this library.  No counterpart in the reference.
+ */
+int magi_attn_fwd_static_scratch(const magi_attn_args* args, void* stream);
+
+/*
  * Fused QK-norm + partial non-interleaved rotary + bf16 cast + KV-cache write, one pass.
  *
  * Stands in for get_q / get_k / get_v / get_kv after the linear layers

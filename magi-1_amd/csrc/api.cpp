@@ -6,6 +6,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "kernels.h"
 #include "magi_attn.h"
@@ -51,6 +52,31 @@ int compute_units() {
   return cached[dev];
 }
 
+// Scratch memory of magi_attn_fwd_static_scratch: the two words of the measured score bound (and room to spare).  One
+// copy per GPU, held until the process ends; every call on a GPU shares it.
+constexpr int SCRATCH_BYTES = 256;
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device (in host code the array's name is a stand-in, not an address):
+// asked once per device with that device current, then kept.
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[64] = {nullptr};
+int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= 64) return fail(MAGI_ENOSYS, "device index %d beyond the 64 this library keeps scratch pointers for", dev);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    g_scratch_ptr[dev] = ptr;
+  }
+  *out = g_scratch_ptr[dev];
+  return MAGI_OK;
+}
+
 int attn_fwd_impl(const magi_attn_args* p, void* stream, float* workspace);
 
 }  // namespace
@@ -67,6 +93,16 @@ int magi_attn_fwd(const magi_attn_args* p, void* stream) {
   if (!p) return fail(MAGI_EINVAL, "magi_attn_fwd: args is NULL");
   MAGI_CHECK_LAYOUT("magi_attn_fwd", p);
   return attn_fwd_impl(p, stream, p->workspace);
+}
+
+int magi_attn_fwd_static_scratch(const magi_attn_args* p, void* stream) {
+  if (!p) return fail(MAGI_EINVAL, "magi_attn_fwd_static_scratch: args is NULL");
+  MAGI_CHECK_LAYOUT("magi_attn_fwd_static_scratch", p);
+  static_assert(4 * sizeof(float) <= SCRATCH_BYTES, "the measured score bound needs four words");
+  void* ws = nullptr;
+  const int rc = static_scratch(&ws);
+  if (rc != MAGI_OK) return rc;
+  return attn_fwd_impl(p, stream, static_cast<float*>(ws));
 }
 
 }  // extern "C"

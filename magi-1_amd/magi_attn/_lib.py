@@ -107,7 +107,7 @@ class QuantizeArgs(_SizedStructure):
 
 ABI_VERSION = 103  # magi_version() of the library these mirrors were written for
 
-EXPORTS = ("magi_version", "magi_last_error", "magi_launch_count", "magi_attn_fwd",
+EXPORTS = ("magi_version", "magi_last_error", "magi_launch_count", "magi_attn_fwd", "magi_attn_fwd_static_scratch",
            "magi_qk_prologue", "magi_head_norm",
            "magi_apply_rotary", "magi_quantize_fp8", "magi_quantize_fp8_split", "magi_layer_norm", "magi_qkv_proj_prologue", "magi_div_clamp_to_e4m3")
 
@@ -131,6 +131,8 @@ def lib() -> C.CDLL:
         l.magi_last_error.restype = C.c_char_p
         l.magi_attn_fwd.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
         l.magi_attn_fwd.restype = C.c_int
+        l.magi_attn_fwd_static_scratch.argtypes = [C.POINTER(AttnArgs), C.c_void_p]
+        l.magi_attn_fwd_static_scratch.restype = C.c_int
         l.magi_qk_prologue.argtypes = [C.POINTER(PrologueArgs), C.c_void_p]
         l.magi_qk_prologue.restype = C.c_int
         l.magi_head_norm.argtypes = [C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32,

@@ -75,6 +75,7 @@ def range_attention(
     q_tile_rows: int = 0,
     bounded_mfma32: bool = False,
     auto_bound: bool = False,
+    static_scratch: bool = False,
     q_norm: Optional[tuple] = None,
     out: Optional[torch.Tensor] = None,
     return_lse: bool = True,
@@ -99,8 +100,9 @@ def range_attention(
     q_tile_rows: force a workgroup shape (0 = the library's choice); see magi_attn_args.q_tile_rows.
     bounded_mfma32 (with q_prescaled and score_bound): the 32x32x16 form of the bounded kernel, MAGI_ATTN_BOUNDED_MFMA32.
     auto_bound (bf16, instead of score_bound): the library measures max|q| and max|k| in two streaming passes and
-    picks the bounded-score kernel on the device when their product allows it, MAGI_ATTN_AUTO_BOUND (its 16-byte
-    workspace is a fresh tensor).
+    picks the bounded-score kernel on the device when their product allows it, MAGI_ATTN_AUTO_BOUND.  Its 16-byte
+    workspace is a fresh tensor, or with static_scratch the library's own device array (magi_attn_fwd_static_scratch:
+    no allocation at all when `out` is given and return_lse is False; such calls must not overlap on one GPU).
     q_norm: (gamma, beta or None, eps[, norm_kind]): q is the raw projection, normalised per (token, head) row inside
     the kernel (fp32, zero-centred gamma) and scaled by softmax_scale * log2(e); needs score_bound.
     """
@@ -180,7 +182,7 @@ def range_attention(
                | (L.MAGI_ATTN_FP8_FAST_EXP2 if fp8_fast_exp2 else 0) | (L.MAGI_ATTN_BOUNDED_MFMA32 if bounded_mfma32 else 0)
                | (L.MAGI_ATTN_AUTO_BOUND if auto_bound else 0))
     workspace = None
-    if auto_bound:
+    if auto_bound and not static_scratch:
         workspace = torch.empty(4, dtype=torch.float32, device=q.device)  # (alive until the launches are enqueued)
         a.workspace = _ptr(workspace)
     a.score_bound = float(score_bound)
@@ -194,7 +196,8 @@ def range_attention(
         a.q_norm_eps = float(q_norm[2])
         a.q_norm_kind = int(q_norm[3]) if len(q_norm) > 3 else L.MAGI_NORM_LAYERNORM_1P
     with torch.cuda.device(q.device):
-        L.check(L.lib().magi_attn_fwd(C.byref(a), _stream()))
+        entry = L.lib().magi_attn_fwd_static_scratch if static_scratch else L.lib().magi_attn_fwd
+        L.check(entry(C.byref(a), _stream()))
     return out, lse
 
 

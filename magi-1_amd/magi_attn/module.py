@@ -32,6 +32,7 @@ import math
 
 from . import _lib as L
 from .cache import Fp8KVCache, OffloadedKVCache
+from .functional import _measuring_a_bound_pays
 from .functional import (div_clamp_to, head_norm, layer_norm, pow2_scale_for, qk_prologue, qk_prologue_fp8, qkv_proj_prologue,
                          quantize_fp8_split,
                          range_attention)
@@ -277,6 +278,11 @@ class FullyParallelAttention(torch.nn.Module):
         self.attention_dtype = attention_dtype
         self.fp8_fast_exp2 = bool(fp8_fast_exp2)
         self.fused_projection = bool(fused_projection) and not fp8_quant
+        # When the bound that follows from the norm parameters exceeds MAGI_SCORE_BOUND_MAX (it takes the largest gain
+        # on both sides for every element), the core attention has the library MEASURE max|q| max|k| on the actual
+        # rows (MAGI_ATTN_AUTO_BOUND), which is far smaller for gains that vary across features.  None: where the two
+        # passes are small beside the attention; True / False: always / never.
+        self.measure_bound_above_limit: Optional[bool] = None
         # forward() has the prologue fold softmax_scale * log2(e) into q ahead of q's one rounding to bf16 and tells
         # the attention kernel so (no per-score multiply there); get_q / get_qkv return q unscaled, as the reference
         self._q_premul = kv_channels ** -0.5 * math.log2(math.e)
@@ -567,15 +573,16 @@ class FullyParallelAttention(torch.nn.Module):
 
     def core_attention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, bs: int,
                        meta_args: ModelMetaArgs, out: Optional[torch.Tensor] = None,
-                       q_prescaled: bool = False, score_bound: float = 0.0) -> torch.Tensor:
+                       q_prescaled: bool = False, score_bound: float = 0.0, auto_bound: bool = False) -> torch.Tensor:
         """query [(sq b), Hq, D], key / value [(sk b), Hkv, D] -> [(sq b), Hq, D]; dit_module.py:1023-1066.
         bs > 1 only occurs with one range per batch row (asserted there too).  `out` (bs == 1 only) is a
         destination view, possibly in the grouped layout of range_attention.  q_prescaled: query carries
-        softmax_scale * log2(e); score_bound: see range_attention."""
+        softmax_scale * log2(e); score_bound, auto_bound: see range_attention."""
         p = meta_args.core_attn_params
         if bs == 1:
             out, _ = range_attention(query, key, value, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                     out=out, return_lse=False, q_prescaled=q_prescaled, score_bound=score_bound)
+                                     out=out, return_lse=False, q_prescaled=q_prescaled, score_bound=score_bound,
+                                     auto_bound=auto_bound)
             return out
         if meta_args.denoising_range_num > 1:
             raise ValueError("bs > 1 with several denoising ranges is not a layout the pipeline produces")
@@ -658,11 +665,26 @@ class FullyParallelAttention(torch.nn.Module):
         # the incoming table already is the [sin | cos] layout the prologue takes
         rope = rotary_pos_emb if (rotary_pos_emb.dtype == torch.float32 and rotary_pos_emb.is_contiguous()) else None
         bound_core = self.score_bounds(rotary_pos_emb.shape[-1] // 2)[0]
+        core_bound_kw = {"score_bound": bound_core}  # (above the limit: the online-softmax kernel, unless measured)
+        measured = False
+        if not (0.0 < bound_core <= L.MAGI_SCORE_BOUND_MAX) and self.attention_dtype == "bf16" and hidden_states.shape[1] == 1:
+            p_ = meta_args.core_attn_params
+            n_q = hidden_states.shape[0]
+            measured = self.measure_bound_above_limit
+            if measured is None:
+                shape_q = torch.empty(n_q, self.num_attention_heads, 128, dtype=torch.bfloat16, device="meta")
+                shape_k = torch.empty(max(int(p_.max_seqlen_k), n_q), self.num_query_groups_per_partition, 128,
+                                      dtype=torch.bfloat16, device="meta")
+                measured = _measuring_a_bound_pays(shape_q, shape_k, p_.q_range.shape[0], p_.max_seqlen_q, p_.max_seqlen_k)
+            if measured:
+                core_bound_kw = {"auto_bound": True}
         # which attention kernels this forward selects (diagnostics; the choice follows from the norm parameters)
         bounded = lambda b: "bounded-score, 64 rows per wavefront" if 0.0 < b <= L.MAGI_SCORE_BOUND_MAX \
             else "online softmax, 32 rows per wavefront"
         self.last_forward_kernels = {
-            "core": "fp8" if self.attention_dtype == "fp8" else bounded(bound_core), "core_score_bound": bound_core,
+            "core": "fp8" if self.attention_dtype == "fp8" else
+            ("measured bound: bounded-score or online softmax, chosen on the device" if measured else bounded(bound_core)),
+            "core_score_bound": bound_core,
             "cross": bounded(self.score_bounds()[1] if hidden_states.shape[1] == 1 else float("inf")),
             "cross_score_bound": self.score_bounds()[1]}
         bs = hidden_states.shape[1]
@@ -716,7 +738,7 @@ class FullyParallelAttention(torch.nn.Module):
         elif not use_cache:
             q, kv, qx_raw = project()
             core = self.core_attention(q, kv[..., :D], kv[..., D:], bs, meta_args, out=core_dst, q_prescaled=True,
-                                       score_bound=bound_core)
+                                       **core_bound_kw)
         else:
             if bs != 1 or inference_params.max_batch_size != 1:
                 raise ValueError("the cached path runs at batch 1 (as the reference pipeline does)")
@@ -749,11 +771,11 @@ class FullyParallelAttention(torch.nn.Module):
                 kc, vc = cache[:split, :, :D], cache[:split, :, D:]
                 if tail is None:
                     core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
-                                              out=core_dst, return_lse=False, q_prescaled=True, score_bound=bound_core)
+                                              out=core_dst, return_lse=False, q_prescaled=True, **core_bound_kw)
                 else:
                     core, _ = range_attention(q, kc, vc, p.q_range, p.k_range, p.max_seqlen_q, p.max_seqlen_k,
                                               k2=tail[:, :, :D], v2=tail[:, :, D:], k_split=split, out=core_dst,
-                                              return_lse=False, q_prescaled=True, score_bound=bound_core)
+                                              return_lse=False, q_prescaled=True, **core_bound_kw)
                 persisted = n_keep
             finally:
                 if offloaded is not None:  # the persisted rows go back to the host behind the attention launch

@@ -407,6 +407,60 @@ def test_layer_follows_rewritten_norm_parameters_and_falls_back_above_the_bound(
     assert "bounded" in layer.last_forward_kernels["core"] and "online" in layer.last_forward_kernels["cross"]
 
 
+def test_layer_measures_the_bound_when_the_parameter_bound_is_too_loose(dev):
+    """Gains that vary across features: the bound that follows from the norm parameters takes the largest gain for
+    every element (here 3 on one feature of q and of k: 148, far above MAGI_SCORE_BOUND_MAX), the rows themselves are
+    hardly longer than with unit gains (measured bound about 30).  With measure_bound_above_limit the core attention measures max|q| max|k| and
+    the bounded-score kernel runs after all: same launches as a call with a stated bound (2 passes + 2 kernels more
+    than the plain launch), parity with the oracle.  With uniform gains of 2 the measured bound (66) is above the
+    limit too and the online-softmax kernel runs behind the measurement: bit-identical to the forward without it."""
+    hidden, Hq, Hkv, D = 256, 6, 2, 128
+    layer = _make_layer(dev, hidden, Hq, Hkv, seed=13)
+    sd = {k_: v_.clone() for k_, v_ in layer.state_dict().items()}
+    for nm in ("q_layernorm", "k_layernorm"):
+        w = torch.zeros(D, device=dev)
+        w[5] = 2.0
+        sd[nm + ".weight"], sd[nm + ".bias"] = w, torch.zeros(D, device=dev)
+    layer.load_state_dict(sd)
+    assert layer.score_bounds()[0] > 2 * M.MAGI_SCORE_BOUND_MAX
+    assert layer.measure_bound_above_limit is None     # (the passes do not pay on a launch this small: plain launch)
+    _cacheless_forward_vs_oracle(layer, dev, 6, tol=4e-2)
+    assert "online" in layer.last_forward_kernels["core"]
+    layer.measure_bound_above_limit = True
+    before = MOD.L.lib().magi_launch_count()
+    _cacheless_forward_vs_oracle(layer, dev, 6, tol=4e-2)
+    with_measurement = MOD.L.lib().magi_launch_count() - before
+    assert "measured" in layer.last_forward_kernels["core"]
+    layer.measure_bound_above_limit = False
+    before = MOD.L.lib().magi_launch_count()
+    _cacheless_forward_vs_oracle(layer, dev, 6, tol=4e-2)
+    assert with_measurement == MOD.L.lib().magi_launch_count() - before + 4
+    # uniform gains of 2: measured 66 > 64, so the measurement ends in the online-softmax kernel
+    sd["q_layernorm.weight"] = torch.full((D,), 1.0, device=dev)
+    sd["k_layernorm.weight"] = torch.full((D,), 1.0, device=dev)
+    layer.load_state_dict(sd)
+    outs = []
+    for flag in (False, True):
+        layer.measure_bound_above_limit = flag
+        from magi_attn.rope import LearnableRotaryEmbeddingCat
+        g = torch.Generator().manual_seed(2)
+        fr, H, W, dn = 2, 3, 4, 2
+        L_ = fr * H * W
+        hs = torch.randn(dn * L_, 1, hidden, generator=g).bfloat16().to(dev)
+        y = (torch.randn(8, hidden, generator=g) * 0.5).bfloat16().to(dev)
+        mask = torch.tensor([[1.0] * 8, [0.0] * 8]).view(dn, 1, 1, 8)
+        meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=0, denoising_range_num=dn,
+                               range_num=dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=False,
+                               distill_nearly_clean_chunk=False, clip_token_nums=L_, enable_cuda_graph=False,
+                               core_attn_params=P.build_core_attn_params(R.q_ranges_from_chunks(dn, L_).to(dev),
+                                                                         R.generate_kv_range_for_uncondition(dn, L_).to(dev), L_),
+                               cross_attn_params=P.build_cross_attn_params(mask.to(dev), L_, 8))
+        rope = LearnableRotaryEmbeddingCat(128, device=dev).get_embed_for_forward(dn * fr, H, W, 0, dn)
+        with torch.no_grad():
+            outs.append(layer(hs, y, None, rope, meta)[0])
+    assert torch.equal(outs[0], outs[1])
+
+
 def test_layer_batched_cacheless_pass(dev):
     """The unconditional pass of classifier-free guidance: chunks become batch rows, tokens are
     ordered (position, batch), every row attends to itself only, no cache."""

@@ -26,18 +26,28 @@ __global__ __launch_bounds__(256) void row_norm_max_kernel(const char* __restric
   const long rows = (long)T * H;
   const long step = (long)gridDim.x * 16;
   unsigned best = 0u;
-  for (long r = (long)blockIdx.x * 16 + (threadIdx.x >> 4); r < rows; r += step) {
-    const long t = r / H;
-    const int h = (int)(r - t * H);
-    const bf16x8 v = *(const bf16x8*)(x + t * stride_t + (long)h * stride_h + sub * 16);
-    float s = 0.f;
+  // four rows in flight per 16-lane group (a row index past the end is clamped to the last row: a maximum does not
+  // mind seeing a row twice)
+  for (long r = (long)blockIdx.x * 16 + (threadIdx.x >> 4); r < rows; r += 4 * step) {
+    bf16x8 v[4];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) s += (float)v[e] * (float)v[e];
-    s += __shfl_xor(s, 1);
-    s += __shfl_xor(s, 2);
-    s += __shfl_xor(s, 4);
-    s += __shfl_xor(s, 8);
-    best = max(best, __float_as_uint(s));
+    for (int u = 0; u < 4; ++u) {
+      const long ru = min(r + u * step, rows - 1);
+      const long t = ru / H;
+      const int h = (int)(ru - t * H);
+      v[u] = *(const bf16x8*)(x + t * stride_t + (long)h * stride_h + sub * 16);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      float s = 0.f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) s += (float)v[u][e] * (float)v[u][e];
+      s += __shfl_xor(s, 1);
+      s += __shfl_xor(s, 2);
+      s += __shfl_xor(s, 4);
+      s += __shfl_xor(s, 8);
+      best = max(best, __float_as_uint(s));
+    }
   }
   best = max(best, (unsigned)__shfl_xor((int)best, 16));
   best = max(best, (unsigned)__shfl_xor((int)best, 32));

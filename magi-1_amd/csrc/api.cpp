@@ -70,7 +70,8 @@ int static_scratch(void** out) {
   if (!g_scratch_ptr[dev]) {
     void* ptr = nullptr;
     e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || !ptr) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (!ptr) return fail(MAGI_EHIP, "hipGetSymbolAddress(scratch) returned no address");
     g_scratch_ptr[dev] = ptr;
   }
   *out = g_scratch_ptr[dev];

@@ -86,6 +86,68 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
     return;
   }
 
+  // ---- K/V tile loader: wave w fills rows 4 * (w + 4 j) .. +3; lane l sits at row +(l >> 4), slot l & 15 ----
+  const long ks_t = a.ks_t, vs_t = a.vs_t;
+  const int k_split = a.k_split;
+  const long k2_delta = a.k2 ? (a.k2 - a.k) - (long)k_split * ks_t : 0;
+  const long v2_delta = a.v2 ? (a.v2 - a.v) - (long)k_split * vs_t : 0;
+  const char* const kcolp = a.k + (long)wi.kvh * a.ks_h;
+  const char* const vcolp = a.v + (long)wi.kvh * a.vs_h;
+
+  auto issue_mat = [&](int k0, unsigned char* tile_base, bool is_v) __attribute__((always_inline)) {
+    unsigned char* dst = tile_base + w * 1024;
+    const long st = is_v ? vs_t : ks_t;
+    const char* colp = is_v ? vcolp : kcolp;
+    const long d2 = is_v ? v2_delta : k2_delta;
+    // the lane geometry is re-derived from an opaque copy of the lane index at every call, so that nothing of it
+    // occupies registers across the main loop
+    int lane = l;
+    asm volatile("" : "+v"(lane));
+    const int lr = lane >> 4, sl = lane & 15;
+    // logical 16-byte chunk that belongs at this lane's fixed LDS slot.  Row r of a tile keeps chunk c at
+    //   K: c ^ (r & 15)        (ds_read_b128 down 16 rows: 16 different chunks)
+    //   V: c ^ ((r & 7) << 1)  (transposing reads of 32 bytes from each of 8 rows: 8 different 32-byte slots)
+    // and r = 4 (w + 4 j) + lr, so r & 15 = 4 w + lr and r & 7 = 4 (w & 1) + lr whatever j.
+    const int chunk = is_v ? (sl ^ ((4 * (w & 1) + lr) << 1)) : (sl ^ (4 * w + lr));
+    const bool interior = (k0 + BN <= ke) && (k0 + BN <= k_split || k0 >= k_split);
+    if (interior) {
+      // buffer-addressed direct loads: tile base in the resource descriptor, one 32-bit lane offset, the row
+      // group of load j in the scalar offset
+      const char* b = colp + (long)k0 * st + (k0 >= k_split ? d2 : 0);
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)b, 0, 0x7fffffff, 0x00020000);
+      const unsigned voff = (unsigned)(4 * w + lr) * (unsigned)st + (unsigned)(chunk * 16);
+#pragma unroll
+      for (int j = 0; j < LOADS; ++j)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * NW * 1024), 16, voff,
+                                                 (int)((unsigned)(4 * NW * j) * (unsigned)st), 0, 0);
+    } else {
+      // Ragged end of the range, or a tile that straddles the two key segments: per-lane rows, clamped to the last
+      // valid key, each lane reading through the descriptor of the segment its row lives in.  Still buffer loads
+      // (a global_load ... lds anywhere in the kernel counts as a possible FLAT access to LDS, after which the
+      // compiler waits for ALL outstanding LDS reads in front of every MFMA instead of counting them).
+      const char* b1 = colp + (long)k0 * st;  // row k0 of the first segment, of the second: (rows >= k_split only)
+      const char* b2 = b1 + d2;
+      const __amdgpu_buffer_rsrc_t rs1 = __builtin_amdgcn_make_buffer_rsrc((void*)b1, 0, 0x7fffffff, 0x00020000);
+      const __amdgpu_buffer_rsrc_t rs2 = __builtin_amdgcn_make_buffer_rsrc((void*)b2, 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+      for (int j = 0; j < LOADS; ++j) {
+        const int row = min(k0 + 4 * w + lr + 4 * NW * j, ke - 1);
+        const unsigned voff = (unsigned)(row - k0) * (unsigned)st + (unsigned)(chunk * 16);
+        if (row < k_split)
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs1, LDS_PTR(void, dst + j * NW * 1024), 16, voff, 0, 0, 0);
+        else
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs2, LDS_PTR(void, dst + j * NW * 1024), 16, voff, 0, 0, 0);
+      }
+    }
+  };
+
+  // The first tile (the LAST one of the key range, see below) is requested before q is loaded and normalised, so that
+  // the two latencies overlap: it matters where a workgroup sees few tiles (the text cross attention).
+  const int n_tiles = (ke - ks + BN - 1) / BN;
+  const int last = n_tiles - 1;
+  issue_mat(ks + last * BN, sK0, false);
+  issue_mat(ks + last * BN, sV0, true);
+
   // ---- Q fragments (B operand of S^T = K Q^T): lane (n, g) holds Q[row 16 qb + n][32 kk + 8 g .. +8] ----
   bf16x8 qf[4][4];
 #pragma unroll
@@ -156,61 +218,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
     __builtin_amdgcn_sched_barrier(0);
   }
 
-  // ---- K/V tile loader: wave w fills rows 4 * (w + 4 j) .. +3; lane l sits at row +(l >> 4), slot l & 15 ----
-  const long ks_t = a.ks_t, vs_t = a.vs_t;
-  const int k_split = a.k_split;
-  const long k2_delta = a.k2 ? (a.k2 - a.k) - (long)k_split * ks_t : 0;
-  const long v2_delta = a.v2 ? (a.v2 - a.v) - (long)k_split * vs_t : 0;
-  const char* const kcolp = a.k + (long)wi.kvh * a.ks_h;
-  const char* const vcolp = a.v + (long)wi.kvh * a.vs_h;
-
-  auto issue_mat = [&](int k0, unsigned char* tile_base, bool is_v) __attribute__((always_inline)) {
-    unsigned char* dst = tile_base + w * 1024;
-    const long st = is_v ? vs_t : ks_t;
-    const char* colp = is_v ? vcolp : kcolp;
-    const long d2 = is_v ? v2_delta : k2_delta;
-    // the lane geometry is re-derived from an opaque copy of the lane index at every call, so that nothing of it
-    // occupies registers across the main loop
-    int lane = l;
-    asm volatile("" : "+v"(lane));
-    const int lr = lane >> 4, sl = lane & 15;
-    // logical 16-byte chunk that belongs at this lane's fixed LDS slot.  Row r of a tile keeps chunk c at
-    //   K: c ^ (r & 15)        (ds_read_b128 down 16 rows: 16 different chunks)
-    //   V: c ^ ((r & 7) << 1)  (transposing reads of 32 bytes from each of 8 rows: 8 different 32-byte slots)
-    // and r = 4 (w + 4 j) + lr, so r & 15 = 4 w + lr and r & 7 = 4 (w & 1) + lr whatever j.
-    const int chunk = is_v ? (sl ^ ((4 * (w & 1) + lr) << 1)) : (sl ^ (4 * w + lr));
-    const bool interior = (k0 + BN <= ke) && (k0 + BN <= k_split || k0 >= k_split);
-    if (interior) {
-      // buffer-addressed direct loads: tile base in the resource descriptor, one 32-bit lane offset, the row
-      // group of load j in the scalar offset
-      const char* b = colp + (long)k0 * st + (k0 >= k_split ? d2 : 0);
-      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)b, 0, 0x7fffffff, 0x00020000);
-      const unsigned voff = (unsigned)(4 * w + lr) * (unsigned)st + (unsigned)(chunk * 16);
-#pragma unroll
-      for (int j = 0; j < LOADS; ++j)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * NW * 1024), 16, voff,
-                                                 (int)((unsigned)(4 * NW * j) * (unsigned)st), 0, 0);
-    } else {
-      // Ragged end of the range, or a tile that straddles the two key segments: per-lane rows, clamped to the last
-      // valid key, each lane reading through the descriptor of the segment its row lives in.  Still buffer loads
-      // (a global_load ... lds anywhere in the kernel counts as a possible FLAT access to LDS, after which the
-      // compiler waits for ALL outstanding LDS reads in front of every MFMA instead of counting them).
-      const char* b1 = colp + (long)k0 * st;  // row k0 of the first segment, of the second: (rows >= k_split only)
-      const char* b2 = b1 + d2;
-      const __amdgpu_buffer_rsrc_t rs1 = __builtin_amdgcn_make_buffer_rsrc((void*)b1, 0, 0x7fffffff, 0x00020000);
-      const __amdgpu_buffer_rsrc_t rs2 = __builtin_amdgcn_make_buffer_rsrc((void*)b2, 0, 0x7fffffff, 0x00020000);
-#pragma unroll
-      for (int j = 0; j < LOADS; ++j) {
-        const int row = min(k0 + 4 * w + lr + 4 * NW * j, ke - 1);
-        const unsigned voff = (unsigned)(row - k0) * (unsigned)st + (unsigned)(chunk * 16);
-        if (row < k_split)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs1, LDS_PTR(void, dst + j * NW * 1024), 16, voff, 0, 0, 0);
-        else
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs2, LDS_PTR(void, dst + j * NW * 1024), 16, voff, 0, 0, 0);
-      }
-    }
-  };
-
   // ---- per-lane LDS read bases ----
   // K as A operand: row = 16 kb + n, 16-byte chunk 4 kk + g, kept at (4 kk + g) ^ n = (4 kk) ^ (g ^ n)
   //   -> off = base_k ^ (kk << 6), + 16 kb rows
@@ -226,8 +233,6 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   float l_run[4] = {0.f, 0.f, 0.f, 0.f};  // this lane's share of the row sums, per query block
   const bool wave_on = row0 < qe;
   const f32x4v zero4 = {0.f, 0.f, 0.f, 0.f};
-
-  const int n_tiles = (ke - ks + BN - 1) / BN;
 
   // One 64-key tile for this wave.  The 32 operand fragments of a tile are consumed in this order:
   //   half t = 0, 1:  K(t, kb = 0..1, kk = 0..3)  [scores of 32 keys x 64 queries]   then   V^T(t, db = 0..7)
@@ -255,7 +260,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
 
     f32x4v sc[2][4];  // scores of the current half: [key block][query block]
     u32x4 pf[4];      // their probabilities as the B operand of the PV MFMAs, per query block
-    static_for<0, 32>([&](auto oc) __attribute__((always_inline)) {
+    auto consume = [&](auto oc) __attribute__((always_inline)) {
       constexpr int o = decltype(oc)::value;
       constexpr int t = o >> 4, j = o & 15;
       // ---- softmax of half t (32 keys x 64 queries: 32 values per lane, one query per lane and query block), one
@@ -313,21 +318,22 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
         if constexpr (!(nj >= 8 && nj < 8 + RD)) ring[o % RD] = read_op(std::integral_constant<int, o + RD>{});
       }
       __builtin_amdgcn_sched_barrier(0);
-    });
+    };
+    static_for<0, 16>(consume);
+    // (the ragged tile: a second half without a valid key has nothing to add.  Short key ranges, the text cross
+    // attention with its dozen tiles per workgroup, are where this is noticeable.)
+    if (!decltype(ragged)::value || ke - k0 > 32) static_for<16, 32>(consume);
   };
 
-  const int last = n_tiles - 1;
   // Tile order: the LAST tile of the key range first (it may hold the ragged end, so it runs the copy of the tile
   // body that masks the tail; the order of keys is immaterial to a softmax), then tiles 0 .. n_tiles-2 with the
   // mask-free body, two per loop iteration so that every LDS slot is named statically.  Tile `last` uses slot
   // pair 0, tile j slot pair (j + 1) & 1.
   const std::integral_constant<int, 0> slot0;
   const std::integral_constant<int, 1> slot1;
-  issue_mat(ks + last * BN, sK0, false);
-  issue_mat(ks + last * BN, sV0, true);
   // The accumulators start from zeros the compiler cannot see through: left to fold them into the first tile's
   // MFMAs it allocates that tile's registers differently from the steady-state body and spills two accumulators
-  // there, a round trip to scratch memory for every workgroup.  (Here, behind the tile requests, so that the 128
+  // there, a round trip to scratch memory for every workgroup.  (Here, behind the q fragments, so that the 128
   // registers are not held while q is loaded and normalised: the statement below pins the finished q fragments
   // ahead of them, or the compiler sinks the norm arithmetic to its first use, behind the zeros.)
   asm volatile("" ::"v"(qf[0][0]), "v"(qf[0][1]), "v"(qf[0][2]), "v"(qf[0][3]), "v"(qf[1][0]), "v"(qf[1][1]), "v"(qf[1][2]),

@@ -331,3 +331,39 @@ def test_inference_params_swap_key_value_dict():
     assert torch.equal(ip.key_value_memory_dict[0], want) and torch.equal(ip.key_value_memory_dict[5], want + 1000)
     with pytest.raises(ValueError):
         ip.swap_key_value_dict([0, 1])
+
+
+def test_copying_form_of_the_cache_update_matches_the_reference_semantics():
+    """FullyParallelAttention.adjust_key_and_value_for_inference, the method with the reference's signature for
+    callers that hold a materialised key_and_value (dit_module.py:891-946): pure tensor work, so it runs on the CPU.
+    Against the oracle's list-of-rows model through a schedule with appends, reads without update, the distill form
+    that drops the last chunk, no inference_params at all, and batch 2."""
+    from magi_attn.module import FullyParallelAttention
+    from oracle import magi_oracle as O
+    Hkv, D, L_ = 2, 128, 5
+    for bs in (1, 2):
+        layer = FullyParallelAttention(64, 4, Hkv, layer_number=2, device="cpu")
+        ip = P.InferenceParams(bs, 6 * L_)
+        model = O.KVCacheModel(6 * L_, Hkv, D, max_batch_size=bs)
+        g = torch.Generator().manual_seed(bs)
+        written = 0
+        # (slice_point, chunks, update, distill, fwd_extra_1st_chunk)
+        for sp, dn, update, distill, extra in ((0, 2, True, False, True), (2, 2, False, False, False),
+                                               (2, 2, True, True, False), (3, 3, True, False, False),
+                                               (0, 1, True, False, False)):
+            kv = torch.randn(dn * L_ * bs, Hkv, 2 * D, generator=g).bfloat16()
+            ip.update_kv_cache = update
+            meta = P.ModelMetaArgs(H=1, W=L_, cp_pad_size=None, cp_split_sizes=None, slice_point=sp, denoising_range_num=dn,
+                                   range_num=sp + dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=extra,
+                                   distill_nearly_clean_chunk=distill, clip_token_nums=L_, enable_cuda_graph=False,
+                                   core_attn_params=None, cross_attn_params=None)
+            k, v = layer.adjust_key_and_value_for_inference(kv, ip, meta)
+            k_ref, v_ref = model.adjust(kv, has_inference_params=True, update_kv_cache=update, slice_point=sp,
+                                        clip_token_nums=L_, fwd_extra_1st_chunk=extra, distill_nearly_clean_chunk=distill)
+            assert torch.equal(k, k_ref) and torch.equal(v, v_ref), (bs, sp, dn)
+            if update:
+                written = max(written, (sp + dn - (1 if distill else 0)) * L_ * bs)
+            # (the layer's cache is allocated uninitialised, as the reference's: rows written so far)
+            assert torch.equal(ip.key_value_memory_dict[2][:written], model.mem[:written])
+        k, v = layer.adjust_key_and_value_for_inference(kv, None, meta)
+        assert torch.equal(k, kv[..., :D]) and torch.equal(v, kv[..., D:])

@@ -658,6 +658,35 @@ def test_layers_with_offloaded_caches_match_resident_ones(dev, staging_buffers):
         assert torch.equal(r0, r1)
 
 
+def test_copying_form_of_the_cache_update_with_offloaded_caches(dev):
+    """adjust_key_and_value_for_inference (the reference-shaped method for a materialised key_and_value) on an
+    offloaded cache: the prefix comes through the staging buffer and the appended rows reach the pinned host copy;
+    keys, values and cache rows equal the oracle's model of the reference's tensor."""
+    from magi_attn.cache import KVCacheArena
+    Hkv, D, L_ = 2, 128, 40
+    layer = MOD.FullyParallelAttention(256, 6, Hkv, layer_number=1, device=dev)
+    arena = KVCacheArena(3, 6 * L_, Hkv, device=dev, kv_offload=True, staging_buffers=2)
+    ip = P.InferenceParams(1, 6 * L_)
+    arena.attach(ip)
+    arena.host.zero_()
+    model = O.KVCacheModel(6 * L_, Hkv, D)
+    g = torch.Generator().manual_seed(4)
+    for sp, dn, update, distill in ((0, 2, True, False), (2, 2, False, False), (2, 2, True, True), (3, 3, True, False)):
+        kv = torch.randn(dn * L_, Hkv, 2 * D, generator=g).bfloat16()
+        ip.update_kv_cache = update
+        meta = P.ModelMetaArgs(H=1, W=L_, cp_pad_size=None, cp_split_sizes=None, slice_point=sp, denoising_range_num=dn,
+                               range_num=sp + dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=True,
+                               distill_nearly_clean_chunk=distill, clip_token_nums=L_, enable_cuda_graph=False,
+                               core_attn_params=None, cross_attn_params=None)
+        k, v = layer.adjust_key_and_value_for_inference(kv.to(dev), ip, meta)
+        k_ref, v_ref = model.adjust(kv, has_inference_params=True, update_kv_cache=update, slice_point=sp,
+                                    clip_token_nums=L_, fwd_extra_1st_chunk=True, distill_nearly_clean_chunk=distill)
+        assert torch.equal(k.cpu(), k_ref) and torch.equal(v.cpu(), v_ref), (sp, dn)
+        arena.synchronize()
+        assert torch.equal(arena.host[1], model.mem)
+    assert not arena.host[0].any() and not arena.host[2].any()
+
+
 @pytest.mark.parametrize("fast_exp2", [True, False])
 def test_layer_with_fp8_self_attention_and_fp8_cache(dev, fast_exp2):
     """attention_dtype="fp8": same schedule as above through two layers with identical weights, one bf16 and one

@@ -306,6 +306,78 @@ def test_layer_forward_sequence_with_kv_cache(dev):
                 assert torch.all(d <= want[..., half].abs().amax(dim=-1, keepdim=True) * 2.0 ** -6)
 
 
+def test_reference_forward_written_out_method_by_method(dev):
+    """The body of the reference's forward for cp_strategy "none" (dit_module.py:1166-1171), typed out with this
+    module's methods of the same names: get_kv, get_q, adjust_key_and_value_for_inference, core_attention,
+    cross_attention with get_xqkv.  This is the path a maintainer gets who swaps the class in but keeps a forward of
+    their own; q stays unscaled here and nothing is appended in place.  Step by step against the oracle's layer and
+    cache, and close to what this module's own forward returns (which pre-scales q: another rounding)."""
+    hidden, Hq, Hkv, D = 256, 6, 2, 128
+    fr, H, W = 2, 3, 4
+    L = fr * H * W
+    n_chunks = 6
+    layer = _make_layer(dev, hidden, Hq, Hkv, seed=17)
+    twin = _make_layer(dev, hidden, Hq, Hkv, seed=17)          # same weights: runs the module's own forward
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+    rope_mod = LearnableRotaryEmbeddingCat(128, device=dev)
+    ip, ip_twin = P.InferenceParams(1, n_chunks * L), P.InferenceParams(1, n_chunks * L)
+    cache_ref = O.KVCacheModel(n_chunks * L, Hkv, D)
+    g = torch.Generator().manual_seed(3)
+    #        sp dn update distill extra has_ip
+    steps = [(0, 2, True, False, True, True), (2, 3, False, False, False, True), (2, 3, True, True, False, True),
+             (4, 2, True, False, False, True), (0, 2, False, False, False, False)]
+    for sp, dn, update, distill, extra, has_ip in steps:
+        S = dn * L
+        hs = torch.randn(S, 1, hidden, generator=g).bfloat16()
+        lens = torch.randint(0, 9, (dn,), generator=g)
+        mask = (torch.arange(8)[None] < lens[:, None]).float().view(dn, 1, 1, 8)
+        y = (torch.randn(int(lens.sum()), hidden, generator=g) * 0.5).bfloat16()
+        k_range = R.generate_default_kvrange(sp, dn, L) if has_ip else R.generate_kv_range_for_uncondition(dn, L)
+        q_range = R.q_ranges_from_chunks(dn, L)
+        cross_p = P.build_cross_attn_params(mask.to(dev), L, 8)
+        meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=sp, denoising_range_num=dn,
+                               range_num=sp + dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=extra,
+                               distill_nearly_clean_chunk=distill, clip_token_nums=L, enable_cuda_graph=False,
+                               core_attn_params=P.build_core_attn_params(q_range.to(dev), k_range.to(dev), L),
+                               cross_attn_params=cross_p)
+        rotary_pos_emb = rope_mod.get_embed_for_forward(dn * fr, H, W, sp, dn)
+        ip.update_kv_cache = ip_twin.update_kv_cache = update
+        params = ip if has_ip else None
+        with torch.no_grad():
+            # ---- dit_module.py:1146-1171, line for line in meaning ----
+            sin_emb, cos_emb = rotary_pos_emb.tensor_split(2, -1)
+            batch_size = hs.shape[1]
+            mixed_qqkv = layer.linear_qkv.forward_ln(hs.to(dev))
+            key_and_value = layer.get_kv(mixed_qqkv, cos_emb, sin_emb)
+            query = layer.get_q(mixed_qqkv, cos_emb, sin_emb)
+            key, value = layer.adjust_key_and_value_for_inference(key_and_value, params, meta)
+            core_attn_out = layer.core_attention(query, key, value, batch_size, meta)
+            core_attn_out = core_attn_out.reshape(S, batch_size, Hq * D)       # "(sq b) hn hd -> sq b (hn hd)"
+            xattn_out = layer.cross_attention(mixed_qqkv, y.to(dev), meta.cross_attn_params, layer.get_xqkv)
+            own_core, own_x = twin(hs.to(dev), y.to(dev), ip_twin if has_ip else None, rotary_pos_emb, meta)
+        assert query.shape == (S, Hq, D) and key_and_value.shape == (S, Hkv, 2 * D) and xattn_out.shape == (S, 1, Hq * D)
+        core_ref, xo_ref = _oracle_layer(layer, hs, y, O.rope_for_forward(dn * fr, H, W, sp, dn), sp, L,
+                                         k_range.numpy(), q_range.numpy(), cache_ref, update, distill, extra,
+                                         cross_p.cu_seqlens_q.cpu(), cross_p.cu_seqlens_kv.cpu(), has_ip)
+        for a, b, nm in ((core_attn_out, core_ref, "core"), (xattn_out, xo_ref, "xattn")):
+            err = (a.float().cpu() - b.float()).abs().max().item()
+            assert err <= 2e-2 and _cosine(a, b) >= 0.9999, f"step {(sp, dn, update, distill, extra)} {nm}: {err}"
+        assert (core_attn_out.float() - own_core.float()).abs().max().item() <= 2e-2
+        assert (xattn_out.float() - own_x.float()).abs().max().item() <= 2e-2
+        if has_ip and (extra or sp > 0) and update:
+            keep = S - L if distill else S
+            rows = slice(sp * L, sp * L + keep)
+            assert torch.equal(ip.key_value_memory_dict[3][rows], ip_twin.key_value_memory_dict[3][rows])  # same prologue
+            got, want = ip.key_value_memory_dict[3][rows].float().cpu(), cache_ref.mem[rows].float()
+            for half in (slice(0, D), slice(D, 2 * D)):
+                d = (got[..., half] - want[..., half]).abs()
+                assert torch.all(d <= want[..., half].abs().amax(dim=-1, keepdim=True) * 2.0 ** -6)
+    # get_qkv: the three pieces of the same prologue
+    with torch.no_grad():
+        q3, k3, v3 = layer.get_qkv(mixed_qqkv, cos_emb, sin_emb)
+    assert torch.equal(q3, query) and torch.equal(k3, key_and_value[..., :D]) and torch.equal(v3, key_and_value[..., D:])
+
+
 def _cacheless_forward_vs_oracle(layer, dev, seed, tol=2e-2):
     """One cache-less batch-1 forward of two chunks (one of them without text) against the oracle's layer."""
     from magi_attn.rope import LearnableRotaryEmbeddingCat

@@ -279,14 +279,22 @@ def test_randomised_shapes_ranges_strides_and_splits(dev):
             split = int(rng.integers(0, Tk + 1))
             kw = dict(k2=kd[split:], v2=vd[split:], k_split=split)  # same strides as the first segment
             kd, vd = kd[:split], vd[:split]
-        out, lse = M.range_attention(q.to(dev), kd, vd, tq, tk, int(ql.max()), q_prescaled=prescaled, **kw)
         cov = torch.tensor(covered, device=dev)
-        if torch.count_nonzero(ref).item() == 0:  # every range of this case is empty
-            assert torch.count_nonzero(out).item() == 0
-        else:
-            _cmp(out[cov], ref[torch.tensor(covered)], f"case {case}")
-        assert torch.count_nonzero(out[~cov]).item() == 0, f"case {case}: uncovered rows written"
-        assert torch.isfinite(out).all()
+        # every kernel that can serve the call: the online softmax, the bounded-score kernel behind a stated bound
+        # (Cauchy-Schwarz on the tensors themselves) and behind the bound the library measures, and its 32x32x16 form
+        factor = 1.0 if prescaled else 128 ** -0.5 * math.log2(math.e)
+        bound = 1.01 * factor * q.float().norm(dim=-1).max().item() * k.float().norm(dim=-1).max().item()
+        kernels = [("online", {}), ("bounded", {"score_bound": bound}), ("measured", {"auto_bound": True})]
+        if prescaled:
+            kernels.append(("bounded-mfma32", {"score_bound": bound, "bounded_mfma32": True}))
+        for name, choice in kernels:
+            out, lse = M.range_attention(q.to(dev), kd, vd, tq, tk, int(ql.max()), q_prescaled=prescaled, **kw, **choice)
+            if torch.count_nonzero(ref).item() == 0:  # every range of this case is empty
+                assert torch.count_nonzero(out).item() == 0
+            else:
+                _cmp(out[cov], ref[torch.tensor(covered)], f"case {case} {name}")
+            assert torch.count_nonzero(out[~cov]).item() == 0, f"case {case} {name}: uncovered rows written"
+            assert torch.isfinite(out).all()
 
 
 def test_repeated_launches_are_bit_identical(dev):

@@ -229,11 +229,13 @@ def test_more_ranges_than_the_in_kernel_ranking_handles(dev):
     Hq, Hkv = 4, 2
     q, k, v = O.synthetic_qkv(int(cu_q[-1]), int(cu_k[-1]), Hq, Hkv, 128, seed=31)
     ref = O.varlen_cross_attention(q, k, v, cu_q, cu_k)
-    out = M.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), torch.tensor(cu_q, device=dev),
-                                   torch.tensor(cu_k, device=dev), int(ql.max()), int(kl.max()))
-    _cmp(out, ref, "300 segments")
     empty_rows = np.concatenate([np.arange(cu_q[i], cu_q[i + 1]) for i in range(n) if kl[i] == 0])
-    assert torch.count_nonzero(out[torch.tensor(empty_rows, device=dev)]).item() == 0
+    # the online-softmax kernel, then the bounded-score kernel behind a stated and behind a measured bound
+    for choice in ({}, {"score_bound": 17.0}, {"auto_bound": True}):
+        out = M.flash_attn_varlen_func(q.to(dev), k.to(dev), v.to(dev), torch.tensor(cu_q, device=dev),
+                                       torch.tensor(cu_k, device=dev), int(ql.max()), int(kl.max()), **choice)
+        _cmp(out, ref, f"300 segments {choice}")
+        assert torch.count_nonzero(out[torch.tensor(empty_rows, device=dev)]).item() == 0
 
 
 def test_randomised_shapes_ranges_strides_and_splits(dev):

@@ -605,6 +605,20 @@ class FullyParallelAttention(torch.nn.Module):
                                score_bound=score_bound)
         return o.view(sq * bs, Hq, D)
 
+    def full_attention(self, bs: int, meta_args: ModelMetaArgs, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, i: int,
+                       score_bound: float = 0.0) -> torch.Tensor:
+        """The rectangle of denoising range i alone: q [rows of range i, Hq, D] against the keys k_range[i] of the
+        whole key axis k / v [(sk), Hkv, D] -> [rows, Hq, D]; dit_module.py:1068-1096 (what the reference's
+        cp_shuffle_overlap strategy calls chunk by chunk, batch 1 only as there).  The range tensors are sliced on the
+        device, so the call does not synchronise."""
+        if bs != 1:
+            raise ValueError("full_attention is defined for batch 1 (as in the reference)")
+        p = meta_args.core_attn_params
+        q_range = (p.q_range[i:i + 1] - p.q_range[i, 0]).contiguous()
+        out, _ = range_attention(q, k, v, q_range, p.k_range[i:i + 1].contiguous(), p.max_seqlen_q, p.max_seqlen_k,
+                                 return_lse=False, score_bound=score_bound)
+        return out
+
     def cross_attention(self, mixed_qqkv: torch.Tensor, key_value_states: torch.Tensor,
                         cross_attn_params: PackedCrossAttnParams, get_xqkv_func: Callable,
                         out: Optional[torch.Tensor] = None) -> torch.Tensor:

@@ -372,6 +372,12 @@ def test_reference_forward_written_out_method_by_method(dev):
             for half in (slice(0, D), slice(D, 2 * D)):
                 d = (got[..., half] - want[..., half]).abs()
                 assert torch.all(d <= want[..., half].abs().amax(dim=-1, keepdim=True) * 2.0 ** -6)
+    # full_attention (dit_module.py:1068-1096): range i on its own gives range i's rows of core_attention
+    with torch.no_grad():
+        for i in range(dn):
+            rows = slice(i * L, (i + 1) * L)
+            o_i = layer.full_attention(1, meta, query[rows], key, value, i)
+            assert torch.equal(o_i, core_attn_out.view(S, Hq, D)[rows]), i
     # get_qkv: the three pieces of the same prologue
     with torch.no_grad():
         q3, k3, v3 = layer.get_qkv(mixed_qqkv, cos_emb, sin_emb)

@@ -541,34 +541,41 @@ class FullyParallelAttention(torch.nn.Module):
         kx = head_norm(kv[..., :D], gk, bk, self.eps)  # strided read, contiguous result
         return qx, kx, kv[..., D:]
 
+    def _full_adjust_key_and_value(self, inference_params: InferenceParams, key_and_value: torch.Tensor,
+                                   meta_args: ModelMetaArgs) -> torch.Tensor:
+        """Appends key_and_value's persistent rows to this layer's cache and returns [cached prefix | key_and_value]
+        (dit_module.py:891-931).  With an offloaded cache the prefix comes through the staging buffer and the appended
+        rows go back to the host."""
+        cache = self._cache(inference_params, key_and_value.dtype)
+        start = meta_args.slice_point * meta_args.clip_token_nums * inference_params.max_batch_size
+        offloaded = cache if isinstance(cache, OffloadedKVCache) else None
+        if offloaded is not None:
+            cache = offloaded.stage(start)
+        clip = 0
+        try:
+            prefix = cache[:start]
+            if inference_params.update_kv_cache:
+                total = key_and_value.size(0)
+                clip = (total - meta_args.clip_token_nums * inference_params.max_batch_size
+                        if meta_args.distill_nearly_clean_chunk else total)
+                if start + clip > cache.shape[0]:
+                    clip = 0
+                    raise ValueError("KV cache overflow")
+                cache[start:start + clip] = key_and_value[:clip]
+            return torch.cat([prefix, key_and_value], dim=0)
+        finally:
+            if offloaded is not None:
+                offloaded.release(start, clip)
+
     def adjust_key_and_value_for_inference(self, key_and_value: torch.Tensor, inference_params: Optional[InferenceParams],
                                            meta_args: ModelMetaArgs):
-        """Copying form with the reference's exact semantics (dit_module.py:891-946), for callers
+        """Copying form with the reference's exact semantics (dit_module.py:933-946), for callers
         that hold a materialised key_and_value.  forward() does not use it: it appends in place."""
         D = self.hidden_size_per_attention_head
         if inference_params is None:
             return key_and_value[..., :D], key_and_value[..., D:]
         if meta_args.extract_prefix_video_feature or meta_args.fwd_extra_1st_chunk or meta_args.slice_point > 0:
-            cache = self._cache(inference_params, key_and_value.dtype)
-            start = meta_args.slice_point * meta_args.clip_token_nums * inference_params.max_batch_size
-            offloaded = cache if isinstance(cache, OffloadedKVCache) else None
-            if offloaded is not None:
-                cache = offloaded.stage(start)
-            clip = 0
-            try:
-                prefix = cache[:start]
-                if inference_params.update_kv_cache:
-                    total = key_and_value.size(0)
-                    clip = (total - meta_args.clip_token_nums * inference_params.max_batch_size
-                            if meta_args.distill_nearly_clean_chunk else total)
-                    if start + clip > cache.shape[0]:
-                        clip = 0
-                        raise ValueError("KV cache overflow")
-                    cache[start:start + clip] = key_and_value[:clip]
-                key_and_value = torch.cat([prefix, key_and_value], dim=0)
-            finally:
-                if offloaded is not None:
-                    offloaded.release(start, clip)
+            key_and_value = self._full_adjust_key_and_value(inference_params, key_and_value, meta_args)
         return key_and_value[..., :D].contiguous(), key_and_value[..., D:].contiguous()
 
     def core_attention(self, query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, bs: int,

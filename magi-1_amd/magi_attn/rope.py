@@ -40,11 +40,45 @@ def build_rotary_table(feat_shape: Sequence[int], bands: torch.Tensor,
     return torch.cat([pos.sin().reshape(n, -1), pos.cos().reshape(n, -1)], dim=-1)
 
 
+def build_fourier_pos_embed(feat_shape: Sequence[int], bands: Optional[torch.Tensor] = None, num_bands: int = 64,
+                            temperature: float = 10000.0, include_grid: bool = False, in_pixels: bool = False,
+                            ref_feat_shape: Optional[Sequence[float]] = None, dtype: torch.dtype = torch.float32,
+                            device=None, **_unused) -> List[torch.Tensor]:
+    """[pos_sin, pos_cos], each feat_shape + [3, num_bands]: the reference's function of this name
+    (dit_module.py:599-667) for the token-index positions the DiT uses (in_pixels=False, dit_model.py:76-78); the
+    pixel-frequency mode is not part of this path."""
+    if in_pixels:
+        raise NotImplementedError("the DiT builds its table with in_pixels=False")
+    if include_grid:
+        raise NotImplementedError("include_grid is not used on this path")
+    if bands is None:
+        bands = freq_bands(num_bands, temperature=temperature, step=1, device=device)
+    table = build_rotary_table(feat_shape, bands, ref_feat_shape)  # [N, 2 * 3 * num_bands] = sin | cos
+    half = table.shape[-1] // 2
+    shape = list(feat_shape) + [len(feat_shape), bands.numel()]
+    return [table[:, :half].reshape(shape).to(dtype), table[:, half:].reshape(shape).to(dtype)]
+
+
+def build_rotary_pos_embed(feat_shape: Sequence[int], bands: Optional[torch.Tensor] = None, dim: int = 64,
+                           temperature: float = 10000.0, in_pixels: bool = False,
+                           ref_feat_shape: Optional[Sequence[float]] = None, dtype: torch.dtype = torch.float32,
+                           device=None, **_unused):
+    """(sin_emb, cos_emb), each [prod(feat_shape), 3 * dim / 8]: dit_module.py:670-717."""
+    sin, cos = build_fourier_pos_embed(feat_shape, bands=bands, num_bands=dim // 8, temperature=temperature,
+                                       in_pixels=in_pixels, ref_feat_shape=ref_feat_shape, dtype=dtype, device=device)
+    n = 1
+    for s in feat_shape:
+        n *= s
+    return sin.reshape(n, -1), cos.reshape(n, -1)
+
+
 class LearnableRotaryEmbeddingCat(torch.nn.Module):
     """Holds the (learnable) bands and builds the table for a [T, H, W] token grid."""
 
-    def __init__(self, dim: int, temperature: float = 10000.0, device=None):
+    def __init__(self, dim: int, temperature: float = 10000.0, device=None, in_pixels: bool = False, **_unused):
         super().__init__()
+        if in_pixels:
+            raise NotImplementedError("the DiT builds its table with in_pixels=False (dit_model.py:76-78)")
         self.dim = dim
         self.temperature = temperature
         self.bands = torch.nn.Parameter(freq_bands(dim // 8, temperature=temperature, step=1, device=device))

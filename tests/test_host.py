@@ -187,6 +187,15 @@ def test_rope_module_matches_oracle():
         b = O.rope_for_forward(T, H, W, sp, dn)
         assert a.shape == (T * H * W, 96) and torch.equal(a, b)
     assert torch.equal(m.get_embed([3, 4, 6]), O.rope_table(3, 4, 6))
+    # the reference's two builder functions by name: (sin, cos) halves of the same table, and their per-axis form
+    sin, cos = RP.build_rotary_pos_embed([3, 4, 6], bands=m.bands.detach(), dim=128)
+    assert sin.shape == cos.shape == (72, 48) and torch.equal(torch.cat([sin, cos], -1), O.rope_table(3, 4, 6))
+    f_sin, f_cos = RP.build_fourier_pos_embed([3, 4, 6], num_bands=16)
+    assert f_sin.shape == (3, 4, 6, 3, 16) and torch.equal(f_sin.reshape(72, 48), sin) and torch.equal(f_cos.reshape(72, 48), cos)
+    assert torch.equal(f_sin[2, 1, 5, 0], torch.sin(2.0 * RP.freq_bands(16)))            # axis 0 is time: position 2
+    with pytest.raises(NotImplementedError):
+        RP.build_rotary_pos_embed([3, 4, 6], in_pixels=True)
+    assert RP.LearnableRotaryEmbeddingCat(128, in_pixels=False).bands.shape == (16,)
 
 
 def test_param_builders():

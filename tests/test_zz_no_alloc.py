@@ -49,7 +49,6 @@ def test_static_scratch_entry_matches_the_workspace_entry(dev):
         cases.append((q.to(dev), k.to(dev), v.to(dev), O.q_ranges_for(dn, L_), O.default_kvrange(sp, dn, L_), L_, (q, k, v)))
     ws = torch.empty(4, dtype=torch.float32, device=dev)
     want = [_call(lib.magi_attn_fwd, dev, q, k, v, qr, kr, mq, ws) for q, k, v, qr, kr, mq, _ in cases]
-    before = torch.cuda.memory_allocated(dev)
     got = []
     for q, k, v, qr, kr, mq, _ in cases:  # back to back, nothing else in between
         got.append(_call(lib.magi_attn_fwd_static_scratch, dev, q, k, v, qr, kr, mq, None))
@@ -57,7 +56,6 @@ def test_static_scratch_entry_matches_the_workspace_entry(dev):
         assert not torch.isnan(o1).any() and torch.equal(o0, o1) and torch.equal(l0, l1)
         ref = O.range_attention(*case[6], case[3], case[4])
         assert (o1.float().cpu() - ref).abs().max().item() <= 2e-2
-    assert torch.cuda.memory_allocated(dev) >= before  # (outputs of this test only; the library has no allocator to ask)
     # without the flag the entry point is magi_attn_fwd
     q, k, v, qr, kr, mq, _ = cases[1]
     plain = M.range_attention(q, k, v, torch.tensor(qr, dtype=torch.int32, device=dev),

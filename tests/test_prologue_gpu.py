@@ -384,6 +384,60 @@ def test_reference_forward_written_out_method_by_method(dev):
     assert torch.equal(q3, query) and torch.equal(k3, key_and_value[..., :D]) and torch.equal(v3, key_and_value[..., D:])
 
 
+@pytest.mark.parametrize("proj_layout", [False, True])
+def test_whole_layer_forward_captured_in_a_graph(dev, proj_layout):
+    """The reference's enable_cuda_graph case at the level of the layer: one FullyParallelAttention.forward on the
+    cached path (input LayerNorm, the projection GEMM, prologue with its in-place cache append, core attention over
+    cache prefix + new rows, text projection, head norm, cross attention) captured into a HIP graph.  Replays on new
+    hidden states and text states, with eager forwards in between, equal the eager results bit for bit."""
+    from magi_attn.rope import LearnableRotaryEmbeddingCat
+    hidden, Hq, Hkv, D = 256, 8, 2, 128
+    fr, H, W = 2, 3, 4
+    L = fr * H * W
+    layer = _make_layer(dev, hidden, Hq, Hkv, seed=23)
+    sp, dn = 2, 2
+    S = dn * L
+    g = torch.Generator().manual_seed(5)
+    hs = torch.randn(S, 1, hidden, generator=g).bfloat16().to(dev)
+    y = (torch.randn(dn * 8, hidden, generator=g) * 0.5).bfloat16().to(dev)
+    meta = P.ModelMetaArgs(H=H, W=W, cp_pad_size=None, cp_split_sizes=None, slice_point=sp, denoising_range_num=dn,
+                           range_num=sp + dn, extract_prefix_video_feature=False, fwd_extra_1st_chunk=True,
+                           distill_nearly_clean_chunk=False, clip_token_nums=L, enable_cuda_graph=True,
+                           core_attn_params=P.build_core_attn_params(R.q_ranges_from_chunks(dn, L).to(dev),
+                                                                     R.generate_default_kvrange(sp, dn, L).to(dev), L),
+                           cross_attn_params=P.build_cross_attn_params(torch.ones(dn, 1, 1, 8).to(dev), L, 8))
+    rope = LearnableRotaryEmbeddingCat(128, device=dev).get_embed_for_forward(dn * fr, H, W, sp, dn)
+    ip = P.InferenceParams(1, 6 * L)
+    ip.update_kv_cache = True
+    ip.key_value_memory_dict[3] = torch.randn(6 * L, Hkv, 2 * D, generator=g).bfloat16().to(dev)
+    run = lambda: layer(hs, y, ip, rope, meta, proj_layout=proj_layout)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            run()  # warm-up outside the capture (norm-parameter caches, side buffers, GEMM workspaces)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            captured = run()
+        captured = captured if isinstance(captured, tuple) else (captured,)
+        for rep in range(3):
+            hs.copy_(torch.randn(S, 1, hidden, generator=g).bfloat16())
+            y.copy_((torch.randn(dn * 8, hidden, generator=g) * 0.5).bfloat16())
+            eager = run()
+            eager = eager if isinstance(eager, tuple) else (eager,)
+            rows = ip.key_value_memory_dict[3][sp * L:(sp + dn) * L].clone()
+            torch.cuda.synchronize()
+            for t in captured:
+                t.fill_(7)
+            ip.key_value_memory_dict[3][sp * L:(sp + dn) * L].zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            for a, b in zip(captured, eager):
+                assert torch.equal(a, b), f"replay {rep}"
+            assert torch.equal(ip.key_value_memory_dict[3][sp * L:(sp + dn) * L], rows)  # the append is replayed too
+
+
 def _cacheless_forward_vs_oracle(layer, dev, seed, tol=2e-2):
     """One cache-less batch-1 forward of two chunks (one of them without text) against the oracle's layer."""
     from magi_attn.rope import LearnableRotaryEmbeddingCat

@@ -289,11 +289,12 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
             if (key >= pe) s_acc[t][v] = -__builtin_inff();
           }
       }
-      float mx = max3(s_acc[0][0], s_acc[0][1], s_acc[0][2]);
+      // (starting from a constant: a maximum of two raw MFMA results first would cost a canonicalising v_max for each)
+      float mx = -__builtin_inff();
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int v = (t == 0 ? 3 : 0); v < 16; v += 2) mx = max3(mx, s_acc[t][v], s_acc[t][v + 1 < 16 ? v + 1 : v]);
+        for (int v = 0; v < 16; v += 2) mx = max3(mx, s_acc[t][v], s_acc[t][v + 1]);
       mx = half_swap_max(mx);
       if constexpr (POW2) {
         // s_acc already holds exponent - m_run + shift; a value above `shift` is a new row maximum

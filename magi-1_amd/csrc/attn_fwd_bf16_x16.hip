@@ -35,7 +35,11 @@ namespace {
 
 constexpr int ROW_BYTES = 256;  // D = 128 bf16
 constexpr int BN = 64;          // keys per LDS tile
-constexpr int TILE_BYTES = BN * ROW_BYTES;
+// A tile in LDS is 16 groups of four rows (what one wave-wide direct load fills: 64 lanes x 16 bytes).  The groups are
+// spaced by a little more than their 1024 bytes, so that consecutive groups start in different banks and the operand
+// reads need no address arithmetic beyond constant offsets (see the read bases below).
+constexpr int K_GROUP = 1024 + 64, V_GROUP = 1024 + 128;
+constexpr int K_TILE_BYTES = (BN / 4) * K_GROUP, V_TILE_BYTES = (BN / 4) * V_GROUP;
 
 typedef float f32x4v __attribute__((ext_vector_type(4)));
 
@@ -55,6 +59,9 @@ __device__ __forceinline__ int swz(int base, int tie) {
 // per-(token, head) norm in fp32 while it is loaded, times the softmax scale, one rounding to bf16.  2: unscaled
 // bf16 q as the reference's callers pass it: multiplied by the softmax scale while it is loaded (a second rounding
 // to bf16: 2^-9 relative per element, the size of the first).
+// order in which the feature blocks of V^T are visited: 0, 4, 1, 5, 2, 6, 3, 7
+constexpr int v_block(int i) { return (i >> 1) + 4 * (i & 1); }
+
 constexpr int Q_AS_IS = 0, Q_NORM = 1, Q_SCALE = 2;
 
 template <int QMODE>
@@ -64,10 +71,10 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   constexpr int RING = 4;               // operand fragments in flight between LDS and the MFMAs
   // K and V double buffered in four separate LDS objects that are only named statically (an operand read then
   // never waits for the direct loads in flight to the other pair of slots)
-  __shared__ __attribute__((aligned(1024))) unsigned char sK0[TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char sV0[TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char sK1[TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char sV1[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sK0[K_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sV0[V_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sK1[K_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sV1[V_TILE_BYTES];
   __shared__ int s_sel;
 
   if (gate_closed(a)) return;
@@ -95,7 +102,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   const char* const vcolp = a.v + (long)wi.kvh * a.vs_h;
 
   auto issue_mat = [&](int k0, unsigned char* tile_base, bool is_v) __attribute__((always_inline)) {
-    unsigned char* dst = tile_base + w * 1024;
+    const int group = is_v ? V_GROUP : K_GROUP;
+    unsigned char* dst = tile_base + w * group;
     const long st = is_v ? vs_t : ks_t;
     const char* colp = is_v ? vcolp : kcolp;
     const long d2 = is_v ? v2_delta : k2_delta;
@@ -104,11 +112,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
     int lane = l;
     asm volatile("" : "+v"(lane));
     const int lr = lane >> 4, sl = lane & 15;
-    // logical 16-byte chunk that belongs at this lane's fixed LDS slot.  Row r of a tile keeps chunk c at
-    //   K: c ^ (r & 15)        (ds_read_b128 down 16 rows: 16 different chunks)
-    //   V: c ^ ((r & 7) << 1)  (transposing reads of 32 bytes from each of 8 rows: 8 different 32-byte slots)
-    // and r = 4 (w + 4 j) + lr, so r & 15 = 4 w + lr and r & 7 = 4 (w & 1) + lr whatever j.
-    const int chunk = is_v ? (sl ^ ((4 * (w & 1) + lr) << 1)) : (sl ^ (4 * w + lr));
+    // logical 16-byte chunk that belongs at this lane's fixed LDS slot.  Row r of a tile (row r & 3 = lr of its
+    // group) keeps chunk c at
+    //   K: c ^ (r & 3)         (ds_read_b128 down 16 rows: four groups 64 bytes apart x four chunks)
+    //   V: c ^ ((r & 3) << 1)  (transposing reads of 32 bytes from each of 8 rows: two groups 128 bytes apart x
+    //                           four 32-byte slots)
+    const int chunk = is_v ? (sl ^ (lr << 1)) : (sl ^ lr);
     const bool interior = (k0 + BN <= ke) && (k0 + BN <= k_split || k0 >= k_split);
     if (interior) {
       // buffer-addressed direct loads: tile base in the resource descriptor, one 32-bit lane offset, the row
@@ -118,7 +127,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
       const unsigned voff = (unsigned)(4 * w + lr) * (unsigned)st + (unsigned)(chunk * 16);
 #pragma unroll
       for (int j = 0; j < LOADS; ++j)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * NW * 1024), 16, voff,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, LDS_PTR(void, dst + j * NW * group), 16, voff,
                                                  (int)((unsigned)(4 * NW * j) * (unsigned)st), 0, 0);
     } else {
       // Ragged end of the range, or a tile that straddles the two key segments: per-lane rows, clamped to the last
@@ -134,9 +143,9 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
         const int row = min(k0 + 4 * w + lr + 4 * NW * j, ke - 1);
         const unsigned voff = (unsigned)(row - k0) * (unsigned)st + (unsigned)(chunk * 16);
         if (row < k_split)
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs1, LDS_PTR(void, dst + j * NW * 1024), 16, voff, 0, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs1, LDS_PTR(void, dst + j * NW * group), 16, voff, 0, 0, 0);
         else
-          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs2, LDS_PTR(void, dst + j * NW * 1024), 16, voff, 0, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rs2, LDS_PTR(void, dst + j * NW * group), 16, voff, 0, 0, 0);
       }
     }
   };
@@ -219,15 +228,17 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   }
 
   // ---- per-lane LDS read bases ----
-  // K as A operand: row = 16 kb + n, 16-byte chunk 4 kk + g, kept at (4 kk + g) ^ n = (4 kk) ^ (g ^ n)
-  //   -> off = base_k ^ (kk << 6), + 16 kb rows
-  const int base_k = n * ROW_BYTES + ((g ^ n) << 4);
+  // K as A operand: row 16 kb + n, 16-byte chunk 4 kk + g, kept at (4 kk + g) ^ (n & 3) = 4 kk + (g ^ (n & 3)) of row
+  // n & 3 of group 4 kb + n / 4: everything but the lane's own part is a constant offset of the read.  The 16 lanes
+  // of one g touch four groups (64 bytes apart in bank terms) x four chunks: all 64 banks once.
+  const int base_k = (n >> 2) * K_GROUP + (n & 3) * ROW_BYTES + ((g ^ (n & 3)) << 4);
   // V^T through the transposing read: the 16-lane group g serves key rows 4 g + r4 (r4 = (l % 16) / 4) of a 16-key
-  // block; lane 4 r4 + c4 of the group points at the four features 16 db + 4 c4 .. +3 of its row, and receives the
-  // four rows' values of feature 16 db + l % 16.  Those 32 bytes of row r are the 16-byte chunks 2 db, 2 db + 1,
-  // kept at (2 db + c4 / 2) ^ ((r & 7) << 1) = (2 db) ^ ((c4 / 2) ^ ((r & 7) << 1))  -> off = base_v ^ (db << 5)
+  // block, i.e. row r4 of group g (+ 4 per key block); lane 4 r4 + c4 of the group points at the four features
+  // 16 db + 4 c4 .. +3 of its row, and receives the four rows' values of feature 16 db + l % 16.  Those 32 bytes of
+  // the row are 32-byte slot db, kept at db ^ r4 = 4 (db / 4) + ((db % 4) ^ r4): one v_xor per value of db % 4,
+  // the rest constant offsets.  Half a wave touches two groups (128 bytes apart in bank terms) x four slots x 32 bytes.
   const int r4 = n >> 2, c4 = n & 3;
-  const int base_v = (4 * g + r4) * ROW_BYTES + ((((c4 >> 1) ^ ((4 * (g & 1) + r4) << 1))) << 4) + ((c4 & 1) << 3);
+  const int base_v = g * V_GROUP + r4 * ROW_BYTES + (r4 << 5) + (c4 << 3);
 
   f32x4v o_acc[8][4];  // [d block][query block]; zeroed below, right ahead of the first tile
   float l_run[4] = {0.f, 0.f, 0.f, 0.f};  // this lane's share of the row sums, per query block
@@ -235,7 +246,8 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   const f32x4v zero4 = {0.f, 0.f, 0.f, 0.f};
 
   // One 64-key tile for this wave.  The 32 operand fragments of a tile are consumed in this order:
-  //   half t = 0, 1:  K(t, kb = 0..1, kk = 0..3)  [scores of 32 keys x 64 queries]   then   V^T(t, db = 0..7)
+  //   half t = 0, 1:  K(t, kb = 0..1, kk = 0..3)  [scores of 32 keys x 64 queries]   then   V^T(t, db = 0, 4, 1, 5,
+  //   2, 6, 3, 7: the two of a pair share their address)
   // each fragment feeding four MFMAs (the query blocks); fragment o is requested RD fragments ahead of its use.
   auto compute_tile = [&](const unsigned char* Kt, const unsigned char* Vt, int k0, auto ragged) __attribute__((always_inline)) {
     auto read_op = [&](auto oc) __attribute__((always_inline)) -> bf16x8 {
@@ -243,12 +255,12 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
       constexpr int t = o >> 4, j = o & 15;
       if constexpr (j < 8) {  // K rows 32 t + 16 kb + n, features 32 kk + 8 g .. +8
         constexpr int kb = j >> 2, kk = j & 3;
-        return *LDS_PTR(const bf16x8, Kt + (swz<(kk << 6), o>(base_k, k0) + (32 * t + 16 * kb) * ROW_BYTES));
+        return *LDS_PTR(const bf16x8, Kt + (base_k + kk * 64 + (8 * t + 4 * kb) * K_GROUP));
       } else {  // V^T: feature block db, the two 16-key blocks of half t
-        constexpr int db = j - 8;
-        const int bv = swz<(db << 5), o>(base_v, k0);
-        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (32 * t) * ROW_BYTES)));
-        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (32 * t + 16) * ROW_BYTES)));
+        constexpr int db = v_block(j - 8);
+        const int bv = swz<((db & 3) << 5), 16 * t + (db & 3)>(base_v, k0) + (db >> 2) * 128;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (8 * t) * V_GROUP)));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16(LDS_PTR(s16x4, Vt + (bv + (8 * t + 4) * V_GROUP)));
         const s16x8 va = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
         return __builtin_bit_cast(bf16x8, va);
       }
@@ -306,7 +318,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
           sc[kb][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[o % RD], qf[qb][kk], kk == 0 ? c0 : sc[kb][qb], 0, 0, 0);
       } else {
         // O^T[d][q] += V^T[d][key] P^T[key][q]
-        constexpr int db = j - 8;
+        constexpr int db = v_block(j - 8);
 #pragma unroll
         for (int qb = 0; qb < 4; ++qb)
           o_acc[db][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ring[o % RD], __builtin_bit_cast(bf16x8, pf[qb]), o_acc[db][qb], 0, 0, 0);

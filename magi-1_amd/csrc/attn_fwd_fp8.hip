@@ -21,7 +21,13 @@ typedef int i32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BN = 64;
 constexpr int ROW_BYTES = 128;  // D = 128 fp8
-constexpr int TILE_BYTES = BN * ROW_BYTES;
+// A tile in LDS is eight groups of eight rows (what one wave-wide direct load fills: 64 lanes x 16 bytes), in key
+// order.  The groups are spaced by a little more than their 1024 bytes and the MFMAs take the keys of a tile in an
+// order that spreads every operand read over the groups (see the read bases below): consecutive groups start 16
+// (K) or 32 (V) bytes further round the banks, so no swizzle is needed and every read address is the lane's base
+// plus a constant.
+constexpr int K_GROUP = 1024 + 16, V_GROUP = 1024 + 32;
+constexpr int K_TILE_BYTES = (BN / 8) * K_GROUP, V_TILE_BYTES = (BN / 8) * V_GROUP;
 constexpr int NW = 4;
 constexpr int BM = 32 * NW;
 constexpr int LOADS = 8 / NW;  // direct loads per wave per matrix per tile (8 rows each)
@@ -35,10 +41,10 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   // then knows that a read of one buffer cannot alias the direct-to-LDS loads in flight to the other and does
   // not make it wait for them (with one array and a run-time buffer index every LDS read waited for vmcnt(0),
   // i.e. for the tile that had just been requested).
-  __shared__ __attribute__((aligned(1024))) unsigned char sK0[TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char sV0[TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char sK1[TILE_BYTES];
-  __shared__ __attribute__((aligned(1024))) unsigned char sV1[TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sK0[K_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sV0[V_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sK1[K_TILE_BYTES];
+  __shared__ __attribute__((aligned(1024))) unsigned char sV1[V_TILE_BYTES];
   __shared__ int s_sel;
 
   const int tid = threadIdx.x;
@@ -83,8 +89,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   // ---- tile loader: wave w fills rows 8*(w + NW*j) .. +7; lane l sits at row +(l >> 3), slot l & 7 ----
   const int lrow = l >> 3, slot = l & 7;
   const int row_in_tile0 = 8 * w + lrow;
-  const int kchunk = slot ^ (4 * (w & 1) + (lrow >> 1));                    // K: chunk ^= (row >> 1) & 7
-  const int vchunk = slot ^ ((((lrow >> 1) & 1) | ((w & 1) << 1)) << 1);    // V: chunk ^= f(row >> 1) << 1
+  const int kchunk = slot, vchunk = slot;  // rows are kept as they are in memory
   const long ks_t = a.ks_t, vs_t = a.vs_t;
   const int k_split = a.k_split;
   const long k2_delta = a.k2 ? (a.k2 - a.k) - (long)k_split * ks_t : 0;
@@ -117,9 +122,9 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
           (void*)(vcol_u + (long)k0 * vs_t + (second ? v2_delta : 0)), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
       for (int j = 0; j < LOADS; ++j) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, LDS_PTR(void, dK + (w + j * NW) * 1024), 16, kvoff,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, LDS_PTR(void, dK + (w + j * NW) * K_GROUP), 16, kvoff,
                                                  (int)((unsigned)(8 * NW * j) * (unsigned)ks_t), 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, LDS_PTR(void, dV + (w + j * NW) * 1024), 16, vvoff,
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, LDS_PTR(void, dV + (w + j * NW) * V_GROUP), 16, vvoff,
                                                  (int)((unsigned)(8 * NW * j) * (unsigned)vs_t), 0, 0);
       }
       return;
@@ -134,22 +139,29 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
 #pragma unroll
     for (int j = 0; j < LOADS; ++j) {
       const int rel = min(row_in_tile0 + 8 * NW * j, pe - 1 - k0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, LDS_PTR(void, dK + (w + j * NW) * 1024), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(kr, LDS_PTR(void, dK + (w + j * NW) * K_GROUP), 16,
                                                (unsigned)rel * (unsigned)ks_t + (unsigned)(kchunk * 16), 0, 0, 0);
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, LDS_PTR(void, dV + (w + j * NW) * 1024), 16,
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(vr, LDS_PTR(void, dV + (w + j * NW) * V_GROUP), 16,
                                                (unsigned)rel * (unsigned)vs_t + (unsigned)(vchunk * 16), 0, 0, 0);
     }
   };
 
   // ---- per-lane LDS read bases ----
-  // K (A operand): row 32t + i, chunks 4kk + 2g + u  ->  (base_k ^ (u << 4) ^ (kk << 6)) + t * 4096
-  const int base_k = i * ROW_BYTES + (((((i >> 1) & 7) ^ (2 * g))) << 4);
-  // V^T via ds_read_b64_tr_b8: in a 16-lane group lane pair (2r', 2r'+1) supplies row r' of 8, lane gets d column l & 15.
-  // Operand slot e = 16t + 4b + r holds key 32t + 8b + 4g + r; read n2 covers t = n2 >> 1, b in {2(n2&1), +1}.
+  // Order of the keys of a tile.  Row i of the score MFMA of half t (t = 0, 1) is key 8 (i & 7) + 4 t + (i >> 3) of
+  // the tile, i.e. row 4 t + (i >> 3) of group i & 7; register v of lane (query, g) of its result is row
+  // i = 8 (v >> 2) + 4 g + (v & 3), i.e. key
+  //     32 g + 8 (v & 3) + 4 t + (v >> 2)                                                             (*)
+  // which is also the key that slot 16 t + v of this lane's 32 slots of the P and V^T operands stands for.
+  // K (A operand): 32 bytes at byte 64 kk + 32 g of that row.  The 16 lanes one ds_read_b128 serves at a time
+  // (i = 0 .. 15 or 16 .. 31, one g) touch eight groups (16 bytes apart in bank terms) x two rows 128 bytes apart: all
+  // 64 banks once.
+  const int base_k = (i & 7) * K_GROUP + (i >> 3) * ROW_BYTES + g * 32;
+  // V^T via ds_read_b64_tr_b8: in a 16-lane group lane pair (2r', 2r'+1) supplies row r' of 8, lane gets d column
+  // l & 15.  Read n2 delivers slots 16 t + 4 b + r for t = n2 >> 1, b = 2 (n2 & 1) + (r' >> 2), r = r' & 3: by (*) row
+  // 4 t + b of group 4 g + r.  The 32 lanes one ds_read_b64 serves at a time touch four groups (32 bytes apart in bank
+  // terms) x two rows x 32 bytes.
   const int lam = l & 15, rp = lam >> 1, dblk = (l >> 4) & 1;
-  const int rho0 = 4 * g + (rp & 3) + 8 * (rp >> 2);
-  const int f_v = (lam >> 2) & 3;
-  const int base_v = rho0 * ROW_BYTES + (((2 * f_v) | dblk) << 4) + (l & 1) * 8;
+  const int base_v = (4 * g + (rp & 3)) * V_GROUP + (rp >> 2) * ROW_BYTES + dblk * 16 + (l & 1) * 8;
 
   f32x16 o_acc[4];
 #pragma unroll
@@ -230,17 +242,17 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
       }
 
       auto read_k = [&](int t, int kk) -> i32x8 {
-        const int o = (base_k ^ (kk << 6)) + t * 4096;
+        const int o = base_k + kk * 64 + t * (4 * ROW_BYTES);
         const i32x4 lo = *LDS_PTR(const i32x4, Kt + o);
-        const i32x4 hi = *LDS_PTR(const i32x4, Kt + (o ^ 16));
+        const i32x4 hi = *LDS_PTR(const i32x4, Kt + (o + 16));
         return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
       };
       auto read_v = [&](int mb) -> i32x8 {
-        const int o = base_v ^ (mb << 5);
+        const int o = base_v + mb * 32;
         i32x2 r[4];
 #pragma unroll
         for (int n2 = 0; n2 < 4; ++n2)
-          r[n2] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(i32x2, Vt + (o + (n2 >> 1) * 4096 + (n2 & 1) * 2048)));
+          r[n2] = __builtin_amdgcn_ds_read_tr8_b64_v2i32(LDS_PTR(i32x2, Vt + (o + (4 * (n2 >> 1) + 2 * (n2 & 1)) * ROW_BYTES)));
         return i32x8{r[0][0], r[0][1], r[1][0], r[1][1], r[2][0], r[2][1], r[3][0], r[3][1]};
       };
 
@@ -285,7 +297,7 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
         for (int t = 0; t < 2; ++t)
 #pragma unroll
           for (int v = 0; v < 16; ++v) {
-            const int key = k0 + 32 * t + 8 * (v >> 2) + 4 * g + (v & 3);
+            const int key = k0 + 32 * g + 8 * (v & 3) + 4 * t + (v >> 2);
             if (key >= pe) s_acc[t][v] = -__builtin_inff();
           }
       }

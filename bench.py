@@ -486,6 +486,33 @@ def mfma_ceiling_leg(dev):
     return out
 
 
+def hbm_ceiling_leg(inp, dev):
+    """What kernels of nothing but 16-byte loads and stores sustain on THIS box's memory, in this process, after the
+    timed region: a copy, a read-only and a write-only pass over ~1 GB (the size of the layer's tensors), 20 launches
+    each.  The streaming kernels of the path (prologue, layer norm, fp8 operand preparation) are reported against the
+    copy rate beside the nominal 8 TB/s.  Same measurement-only helper library as the MFMA ceiling."""
+    import ctypes as C
+
+    path = os.path.join(ROOT, "magi-1_amd", "magi_attn", "libmagi_probe.so")
+    if not os.path.exists(path):
+        return {"error": "libmagi_probe.so is not built (make -C magi-1_amd/csrc)"}
+    lib = C.CDLL(path)
+    if not hasattr(lib, "magi_probe_stream"):
+        return {"error": "libmagi_probe.so predates magi_probe_stream (make -C magi-1_amd/csrc)"}
+    lib.magi_probe_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.POINTER(C.c_float)]
+    lib.magi_probe_stream.restype = C.c_int
+    src, dst = inp["cache"], inp["xout"]  # (xout is scratch by now: nothing reads the cross-attention output afterwards)
+    nbytes = min(src.numel() * src.element_size(), dst.numel() * dst.element_size()) // 16 * 16
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = {"what": "16 bytes per lane, one contiguous piece per workgroup; GB/s counts every byte read and every byte written",
+           "unit": "GB/s", "bytes": nbytes}
+    for name, kind, moved in (("copy", 0, 2 * nbytes), ("read_only", 1, nbytes), ("write_only", 2, nbytes)):
+        ms = C.c_float(0)
+        rc = lib.magi_probe_stream(kind, src.data_ptr(), dst.data_ptr(), nbytes, 20, stream, C.byref(ms))
+        out[name] = {"error": rc} if rc != 0 else {"gbs": round(moved / (ms.value * 1e-3) / 1e9, 1), "ms": round(ms.value, 4)}
+    return out
+
+
 def secondary_legs(inp, dev, steps):
     """Core-attention launches the headline does not time, kernel only, a few steps each: the online-softmax kernel a
     caller gets who neither states a score bound nor lets the library measure one (unscaled q), the bounded kernel
@@ -682,6 +709,16 @@ def main():
             pass
     result["roofline_layer_norm"] = layer_norm_leg(inp, args.steps, traffic.get("layer_norm"))
     result["roofline_layer_norm"]["traffic_source"] = TRAFFIC_SOURCE
+    if not args.no_ceiling:
+        hc = hbm_ceiling_leg(inp, dev)
+        result["hbm_ceiling"] = hc
+        top = hc.get("copy", {}).get("gbs")
+        if top:
+            for key in ("roofline_prologue", "roofline_layer_norm"):
+                result[key]["frac_of_measured_copy"] = round(result[key]["achieved"] / top, 4)
+            prep = result.get("fp8", {}).get("operand_preparation")
+            if prep and "achieved" in prep:
+                prep["frac_of_measured_copy"] = round(prep["achieved"] / top, 4)
     if not args.no_projection:
         result["projection"] = projection_leg(inp, args.steps)
     if args.copy_calibration:

@@ -1,7 +1,8 @@
 /* libmagi_probe: measurement only (loaded by bench.py, never by the product path): the rate of an MFMA-only loop
- * on the current GPU, the per-box ceiling the attention kernels' rates are reported against. */
+ * and of plain streaming kernels on the current GPU, the per-box ceilings the kernels' rates are reported against. */
 #ifndef MAGI_PROBE_H
 #define MAGI_PROBE_H
+#include <stddef.h>
 #include <stdint.h>
 #ifdef __cplusplus
 extern "C" {
@@ -15,6 +16,12 @@ extern "C" {
  * them and returns the average milliseconds per launch and the FLOPs of one launch.  0 on success. */
 int magi_probe_mfma_only(int kind, const uint32_t* operands, float* sink, int rounds, int launches, void* stream,
                          float* ms_per_launch, double* flop_per_launch);
+/* kind 0: copy `bytes` from src to dst; 1: read src only (dst: at least 16 bytes, not written in practice);
+ * 2: write dst only (src unused).  DEVICE pointers, 16-byte aligned, bytes a multiple of 16, 16 bytes per lane.
+ * One warm-up launch and `launches` timed ones back to back on `stream`; average milliseconds per launch.  0 on
+ * success. */
+int magi_probe_stream(int kind, const void* src, void* dst, size_t bytes, int launches, void* stream,
+                      float* ms_per_launch);
 #ifdef __cplusplus
 }
 #endif

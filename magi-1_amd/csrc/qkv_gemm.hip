@@ -49,13 +49,14 @@ __global__ __launch_bounds__(64 * (16 / MB), 1) void qkv_gemm_prologue_kernel(co
   unsigned char* const sW1 = smem + 3 * TILE;
   unsigned char* const sJunk = smem + 4 * TILE;  // 1 KB that nothing reads (destination of the cache-warming loads)
 
-  // ---- which tile: blockIdx % 8 is the XCD; an XCD walks blocks of 8 token tiles x all column tiles, token tile
-  // fastest, so that the ~32 workgroups it runs at a time share 8 X slices and 4 W slices through its L2 ----
+  // ---- which tile: blockIdx % 8 is the XCD.  XCD x owns the token tiles x, x + 8, x + 16, ... (an even share for
+  // every XCD whatever the tile count) and walks them in blocks of 8 x all column tiles, token tile fastest, so that
+  // the ~32 workgroups it runs at a time share 8 X slices and 4 W slices through its L2 ----
   const int xcd = blockIdx.x & 7;
   const int t = blockIdx.x >> 3;
-  const int per_super = 8 * a.n_col_tiles;
-  const int ms = t / per_super, r = t % per_super;
-  const int m_tile = (ms * 8 + xcd) * 8 + (r & 7);
+  const int per_block = 8 * a.n_col_tiles;
+  const int qb = t / per_block, r = t % per_block;
+  const int m_tile = (qb * 8 + (r & 7)) * 8 + xcd;
   const int n_tile = r >> 3;
   if (m_tile >= a.n_row_tiles) return;
   const int m0 = m_tile * BM;
@@ -321,8 +322,8 @@ hipError_t launch_qkv_gemm_prologue(const QkvGemmKernArgs& a_in, hipStream_t str
   const int lds = 4 * TILE + 1024;  // 129 KB of the CU's 160: above the default limit, asked for per launch (a host-side setting)
   hipError_t e = hipFuncSetAttribute((const void*)qkv_gemm_prologue_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
   if (e != hipSuccess) return e;
-  const int supers = (a.n_row_tiles + 63) / 64;
-  const unsigned grid = (unsigned)supers * 8u * 8u * (unsigned)a.n_col_tiles;
+  const int blocks = ((a.n_row_tiles + 7) / 8 + 7) / 8;  // blocks of 8 token tiles per XCD
+  const unsigned grid = (unsigned)blocks * 8u * 8u * (unsigned)a.n_col_tiles;
   hipLaunchKernelGGL(qkv_gemm_prologue_kernel<2>, dim3(grid), dim3(512), lds, stream, a);
   return hipGetLastError();
 }

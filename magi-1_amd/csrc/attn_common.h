@@ -87,7 +87,8 @@ struct WorkItem {
 // blockIdx -> (kv head, range slot, q tile, q head within the GQA group), laid out so that the workgroups an
 // XCD receives (blockIdx % 8) share a KV head and walk the same keys at about the same time (each XCD has its
 // own L2).  Ranges are visited longest key span first (ties by index), ranked here from the device-side list.
-// Every thread of the workgroup must call this (it contains a barrier); s_sel is one int of LDS.
+// Every thread of the workgroup must call this (it contains a barrier); s_sel is LOCATE_WORDS ints of LDS.
+constexpr int LOCATE_WORDS = 4;
 __device__ __forceinline__ WorkItem locate_work(const AttnKernArgs& a, int BM, int tid, int* s_sel) {
   WorkItem wi;
   wi.valid = false;
@@ -106,11 +107,14 @@ __device__ __forceinline__ WorkItem locate_work(const AttnKernArgs& a, int BM, i
   wi.h = (int)(kvh * a.G + hg);
   wi.o_head = a.out_group > 0 ? (long)(wi.h / a.out_group) * a.os_g + (long)(wi.h % a.out_group) * a.os_h
                               : (long)wi.h * a.os_h;
-  int ridx;
+  int qs;
   if (a.n_ranges <= MAX_SORT) {
+    // thread t ranks range t; the one whose rank is this workgroup's slot publishes the range itself (its q rows were
+    // requested together with the key ranges: one memory latency for everything)
     if (tid < a.n_ranges) {
-      int s, e;
+      int s, e, q_s, q_e;
       load_range(a.k_ranges, a.ranges_mode, tid, a.total_k, s, e);
+      load_range(a.q_ranges, a.ranges_mode, tid, a.total_q, q_s, q_e);
       const int my = e - s;
       int rank = 0;
       for (int j = 0; j < a.n_ranges; ++j) {
@@ -119,16 +123,23 @@ __device__ __forceinline__ WorkItem locate_work(const AttnKernArgs& a, int BM, i
         const int lj = ej - sj;
         rank += (lj > my) || (lj == my && j < tid);
       }
-      if (rank == (int)rslot) *s_sel = tid;
+      if (rank == (int)rslot) {
+        s_sel[0] = q_s;
+        s_sel[1] = q_e;
+        s_sel[2] = s;
+        s_sel[3] = e;
+      }
     }
     __syncthreads();
-    ridx = __builtin_amdgcn_readfirstlane(*s_sel);
+    qs = __builtin_amdgcn_readfirstlane(s_sel[0]);
+    wi.qe = __builtin_amdgcn_readfirstlane(s_sel[1]);
+    wi.ks = __builtin_amdgcn_readfirstlane(s_sel[2]);
+    wi.ke = __builtin_amdgcn_readfirstlane(s_sel[3]);
   } else {
-    ridx = a.n_ranges - 1 - (int)rslot;
+    const int ridx = a.n_ranges - 1 - (int)rslot;
+    load_range(a.q_ranges, a.ranges_mode, ridx, a.total_q, qs, wi.qe);
+    load_range(a.k_ranges, a.ranges_mode, ridx, a.total_k, wi.ks, wi.ke);
   }
-  int qs;
-  load_range(a.q_ranges, a.ranges_mode, ridx, a.total_q, qs, wi.qe);
-  load_range(a.k_ranges, a.ranges_mode, ridx, a.total_k, wi.ks, wi.ke);
   wi.q0 = qs + (int)tile * BM;
   wi.valid = wi.q0 < wi.qe;
   return wi;

@@ -67,12 +67,12 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_kernel(const AttnK
   static_assert(!VSINGLE || NSTAGE == 2, "single-V mode: two K slots and one V slot");
   static_assert(!DB || (NSTAGE == 2 && !VSINGLE), "static double buffer: two K slots and two V slots");
   static_assert(DB != VSINGLE, "one of the two tile loops");
-  __shared__ int s_sel;
+  __shared__ int s_sel[LOCATE_WORDS];
 
   if (gate_closed(a)) return;
   const int tid = threadIdx.x;
   // ---- which piece of work is this workgroup? ----
-  const WorkItem wi = locate_work(a, BM, tid, &s_sel);
+  const WorkItem wi = locate_work(a, BM, tid, s_sel);
   if (!wi.valid) return;
   const int h = wi.h, q0 = wi.q0, qe = wi.qe, ks = wi.ks, ke = wi.ke;
   const unsigned kvh = (unsigned)wi.kvh;

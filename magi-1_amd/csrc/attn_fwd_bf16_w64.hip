@@ -68,10 +68,10 @@ __global__ __launch_bounds__(64 * NW, OCC) void attn_fwd_bf16_w64_kernel(const A
   __shared__ __attribute__((aligned(1024))) unsigned char sV0[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char sK1[TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char sV1[TILE_BYTES];
-  __shared__ int s_sel;
+  __shared__ int s_sel[LOCATE_WORDS];
 
   const int tid = threadIdx.x;
-  const WorkItem wi = locate_work(a, BM, tid, &s_sel);
+  const WorkItem wi = locate_work(a, BM, tid, s_sel);
   if (!wi.valid) return;
   const int qe = wi.qe, ks = wi.ks, ke = wi.ke;
 

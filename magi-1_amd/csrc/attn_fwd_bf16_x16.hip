@@ -75,11 +75,11 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_bf16_x16_kernel(const AttnKer
   __shared__ __attribute__((aligned(1024))) unsigned char sV0[V_TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char sK1[K_TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char sV1[V_TILE_BYTES];
-  __shared__ int s_sel;
+  __shared__ int s_sel[LOCATE_WORDS];
 
   if (gate_closed(a)) return;
   const int tid = threadIdx.x;
-  const WorkItem wi = locate_work(a, BM, tid, &s_sel);
+  const WorkItem wi = locate_work(a, BM, tid, s_sel);
   if (!wi.valid) return;
   const int qe = wi.qe, ks = wi.ks, ke = wi.ke;
 

@@ -45,10 +45,10 @@ __global__ __launch_bounds__(64 * NW, 3) void attn_fwd_fp8_kernel(const AttnKern
   __shared__ __attribute__((aligned(1024))) unsigned char sV0[V_TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char sK1[K_TILE_BYTES];
   __shared__ __attribute__((aligned(1024))) unsigned char sV1[V_TILE_BYTES];
-  __shared__ int s_sel;
+  __shared__ int s_sel[LOCATE_WORDS];
 
   const int tid = threadIdx.x;
-  const WorkItem wi = locate_work(a, BM, tid, &s_sel);
+  const WorkItem wi = locate_work(a, BM, tid, s_sel);
   if (!wi.valid) return;
   const int h = wi.h, kvh = wi.kvh, q0 = wi.q0, qe = wi.qe, ks = wi.ks, ke = wi.ke;
   const long o_head = wi.o_head;

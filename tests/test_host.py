@@ -29,6 +29,28 @@ def test_library_loads_and_exports_every_declared_symbol():
         assert hasattr(lib, name), name
 
 
+def test_measurement_library_exports_what_its_header_declares():
+    """libmagi_probe.so (MFMA-only and streaming loops that bench.py reports its ceilings from) is built by the same
+    Makefile; nothing in the package loads it.  No compute call without a GPU: argument checks only."""
+    path = os.path.join(ROOT, "magi-1_amd", "magi_attn", "libmagi_probe.so")
+    assert os.path.exists(path), "build it with `make -C magi-1_amd/csrc`"
+    lib = C.CDLL(path)
+    header = open(os.path.join(ROOT, "magi-1_amd", "csrc", "probe", "magi_probe.h")).read()
+    declared = re.findall(r"\b(magi_probe_\w+)\s*\(", header)
+    assert sorted(set(declared)) == ["magi_probe_mfma_only", "magi_probe_stream"]
+    for name in declared:
+        assert hasattr(lib, name), name
+    lib.magi_probe_stream.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.POINTER(C.c_float)]
+    lib.magi_probe_stream.restype = C.c_int
+    ms = C.c_float(0)
+    assert lib.magi_probe_stream(7, None, None, 1024, 1, None, C.byref(ms)) == -22      # unknown kind
+    assert lib.magi_probe_stream(0, None, None, 1024, 1, None, C.byref(ms)) == -22      # no buffers
+    assert lib.magi_probe_stream(2, None, C.c_void_p(256), 1000, 1, None, C.byref(ms)) == -22  # not a multiple of 16
+    for pkg_file in os.listdir(os.path.join(ROOT, "magi-1_amd", "magi_attn")):
+        if pkg_file.endswith(".py"):
+            assert "magi_probe" not in open(os.path.join(ROOT, "magi-1_amd", "magi_attn", pkg_file)).read(), pkg_file
+
+
 def test_missing_library_is_an_error_not_a_fallback(tmp_path):
     """The library beside the package is the only compute path: when it is not there the first call raises (checked
     in a child process on a copy of the package without its .so; no environment variable redirects the loader)."""

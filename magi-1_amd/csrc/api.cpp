@@ -555,7 +555,7 @@ static int quantize_impl(const magi_quantize_args* p, void* stream, bool always_
   hipError_t e = magi::launch_quantize_fp8(static_cast<const char*>(p->x), p->x_stride_t * 2, p->x_stride_h * 2,
                                            static_cast<char*>(p->y), p->scales, p->T, p->H, p->chunk_tokens, p->premul,
                                            p->pow2_scales, p->n_rows_first, static_cast<char*>(p->y2), p->scales2,
-                                           always_one_launch, static_cast<hipStream_t>(stream), &n_launches);
+                                           always_one_launch, compute_units(), static_cast<hipStream_t>(stream), &n_launches);
   if (e != hipSuccess) return hip_fail(e, "magi_quantize_fp8 launch");
   g_launches.fetch_add((uint64_t)n_launches, std::memory_order_relaxed);
   return MAGI_OK;

@@ -606,7 +606,7 @@ hipError_t launch_attn_fwd_fp8(const AttnKernArgs& a, hipStream_t stream) {
 
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
                                int chunk_tokens, float premul, int pow2_scales, int n_first, char* y2, float* scales2,
-                               bool one_launch, hipStream_t stream, int* n_launches) {
+                               bool one_launch, int compute_units, hipStream_t stream, int* n_launches) {
   const int n_chunks = (T + chunk_tokens - 1) / chunk_tokens;
   const int n = n_chunks * H;
   *n_launches = 0;
@@ -617,8 +617,10 @@ hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, 
   if (n_first < T || (min(chunk_tokens, T) <= 8192 && (n >= 64 || (long)T * H <= 65536))) one_launch = true;
   if (one_launch) {
     if (n_chunks > 65535) return hipErrorInvalidValue;
-    // workgroups per group: towards two per CU over the launch, each slice at least four passes long
-    int share = (512 + n - 1) / n;
+    // workgroups per group: towards one per CU over the launch (every workgroup reads its whole group for the absmax, so
+    // a second one per CU doubles what a CU pulls through its caches: 162 instead of 105 us at the 720p shape), each
+    // slice at least four passes long
+    int share = (compute_units + n - 1) / n;
     share = max(1, min(share, min(16, min(chunk_tokens, T) / (4 * QROWS))));
     hipLaunchKernelGGL(quantize_groups_kernel, dim3(H, n_chunks, share), dim3(QT1), 0, stream, x, x_stride_t, x_stride_h, y,
                        scales, T, H, chunk_tokens, premul, pow2_scales, n_first, y2, scales2);

@@ -127,6 +127,6 @@ hipError_t launch_rotary(const void* x, const float* cos, const float* sin, void
 // *n_launches receives the number of kernels launched.
 hipError_t launch_quantize_fp8(const char* x, long x_stride_t, long x_stride_h, char* y, float* scales, int T, int H,
                                int chunk_tokens, float premul, int pow2_scales, int n_first, char* y2, float* scales2,
-                               bool one_launch, hipStream_t stream, int* n_launches);
+                               bool one_launch, int compute_units, hipStream_t stream, int* n_launches);
 
 }  // namespace magi

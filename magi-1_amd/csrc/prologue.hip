@@ -101,12 +101,17 @@ template <int TPB, bool OUT8>
 __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArgs a) {
   __shared__ float s_par[4][D];  // gq, bq, gk, bk
   const int tid = threadIdx.x;
-  for (int i = tid; i < 4 * D; i += THREADS) {
-    const int which = i / D, e = i % D;
+  // Everything a workgroup needs from memory is requested in one go: the norm parameters (two per thread, on their way
+  // to LDS), the token's rotary row and each row group's first row; the barrier that publishes the parameters is where
+  // they are waited for.  (Parameters, barrier, then the rows: two memory latencies in a workgroup that lives for
+  // little more than that.)
+  float par[4 * D / THREADS];
+#pragma unroll
+  for (int k = 0; k < 4 * D / THREADS; ++k) {
+    const int i = tid + k * THREADS, which = i / D, e = i % D;
     const float* src = which == 0 ? a.gq : which == 1 ? a.bq : which == 2 ? a.gk : a.bk;
-    s_par[which][e] = src ? src[e] : 0.f;
+    par[k] = src ? src[e] : 0.f;
   }
-  __syncthreads();
 
   // The 32 row groups of the workgroup form tok_per_block teams of equal size, one token each, so that layers
   // with few heads (e.g. one rank's share of a head-parallel split: 8 rows per token) still fill the workgroup.
@@ -121,50 +126,76 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
   const int U = a.Hq + (OUT8 ? 1 : 2) * a.Hkv;
   constexpr int ES = OUT8 ? 1 : 2;  // bytes per output element
 
-  {
-    const int s = blockIdx.x * TPB + team;
-    if (s >= a.S) return;
-    float sn[8], cs[8];
-    if (rot_lane && a.rope) {
-      const float* rp = a.rope + (long)(s / a.batch) * (2 * a.R2);
-      const f32x4 s0 = *(const f32x4*)(rp + 8 * j), s1 = *(const f32x4*)(rp + 8 * j + 4);
-      const f32x4 c0 = *(const f32x4*)(rp + a.R2 + 8 * j), c1 = *(const f32x4*)(rp + a.R2 + 8 * j + 4);
+  const int s = blockIdx.x * TPB + team;
+  const bool live = s < a.S;
+  float sn[8], cs[8];
+  if (live && rot_lane && a.rope) {
+    const float* rp = a.rope + (long)(s / a.batch) * (2 * a.R2);
+    const f32x4 s0 = *(const f32x4*)(rp + 8 * j), s1 = *(const f32x4*)(rp + 8 * j + 4);
+    const f32x4 c0 = *(const f32x4*)(rp + a.R2 + 8 * j), c1 = *(const f32x4*)(rp + a.R2 + 8 * j + 4);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        sn[i] = s0[i];
-        sn[4 + i] = s1[i];
-        cs[i] = c0[i];
-        cs[4 + i] = c1[i];
-      }
+    for (int i = 0; i < 4; ++i) {
+      sn[i] = s0[i];
+      sn[4 + i] = s1[i];
+      cs[i] = c0[i];
+      cs[4 + i] = c1[i];
     }
-    char* kvrow = (s < a.n_cache_rows) ? a.kv_out + (long)s * a.kv_stride_t
-                                       : a.kv_tail + (long)(s - a.n_cache_rows) * a.kv_tail_stride_t;
-    for (int u = grp; u < U; u += gpt) {
-      const char* src;
-      char* dst;
-      int kind;  // 0 = q, 1 = k, 2 = v
-      if (u < a.Hq) {
-        kind = 0;
-        src = a.q_raw + (long)s * a.q_raw_stride_t + (long)u * (D * 2);
-        dst = a.q_out + ((long)s * a.Hq + u) * (D * ES);
-      } else if (u < a.Hq + a.Hkv) {
-        kind = 1;
-        const int hh = u - a.Hq;
-        src = a.k_raw + (long)s * a.k_raw_stride_t + (long)hh * (D * 2);
-        dst = kvrow + (long)hh * (OUT8 ? D : 2 * D * 2);
-      } else {
-        kind = 2;
-        const int hh = u - a.Hq - a.Hkv;
-        src = a.v_raw + (long)s * a.v_raw_stride_t + (long)hh * (D * 2);
-        dst = kvrow + (long)hh * (2 * D * 2) + D * 2;
-      }
-      const u32x4 va = *(const u32x4*)(src + ea * 2);
-      const u32x4 vb = *(const u32x4*)(src + eb * 2);
-      if (kind == 2) {
-        *(u32x4*)(dst + ea * 2) = va;
-        *(u32x4*)(dst + eb * 2) = vb;
-        continue;
-      }
+  }
+  const int sc = live ? s : 0;  // (a valid row for the address arithmetic of a team past the end)
+  char* kvrow = (sc < a.n_cache_rows) ? a.kv_out + (long)sc * a.kv_stride_t
+                                      : a.kv_tail + (long)(sc - a.n_cache_rows) * a.kv_tail_stride_t;
+  // row u of the token: 0 = q, 1 = k, 2 = v; where it comes from and where it goes
+  auto locate = [&](int u, const char*& src, char*& dst, int& kind) __attribute__((always_inline)) {
+    if (u < a.Hq) {
+      kind = 0;
+      src = a.q_raw + (long)sc * a.q_raw_stride_t + (long)u * (D * 2);
+      dst = a.q_out + ((long)sc * a.Hq + u) * (D * ES);
+    } else if (u < a.Hq + a.Hkv) {
+      kind = 1;
+      const int hh = u - a.Hq;
+      src = a.k_raw + (long)sc * a.k_raw_stride_t + (long)hh * (D * 2);
+      dst = kvrow + (long)hh * (OUT8 ? D : 2 * D * 2);
+    } else {
+      kind = 2;
+      const int hh = u - a.Hq - a.Hkv;
+      src = a.v_raw + (long)sc * a.v_raw_stride_t + (long)hh * (D * 2);
+      dst = kvrow + (long)hh * (2 * D * 2) + D * 2;
+    }
+  };
+  int u = grp;
+  const char* src = nullptr;
+  char* dst = nullptr;
+  int kind = 0;
+  u32x4 va = {0u, 0u, 0u, 0u}, vb = va;
+  if (live && u < U) {
+    locate(u, src, dst, kind);
+    va = *(const u32x4*)(src + ea * 2);
+    vb = *(const u32x4*)(src + eb * 2);
+  }
+#pragma unroll
+  for (int k = 0; k < 4 * D / THREADS; ++k) {
+    const int i = tid + k * THREADS;
+    s_par[i / D][i % D] = par[k];
+  }
+  __syncthreads();
+  if (!live) return;
+
+  while (u < U) {
+    // the next row of this group is requested before the current one is worked on
+    const int u_next = u + gpt;
+    const char* src_n = nullptr;
+    char* dst_n = nullptr;
+    int kind_n = 0;
+    u32x4 va_n = va, vb_n = vb;
+    if (u_next < U) {
+      locate(u_next, src_n, dst_n, kind_n);
+      va_n = *(const u32x4*)(src_n + ea * 2);
+      vb_n = *(const u32x4*)(src_n + eb * 2);
+    }
+    if (kind == 2) {
+      *(u32x4*)(dst + ea * 2) = va;
+      *(u32x4*)(dst + eb * 2) = vb;
+    } else {
       float x[16];
       unpack8(va, x);
       unpack8(vb, x + 8);
@@ -192,6 +223,12 @@ __global__ __launch_bounds__(THREADS) void prologue_kernel(const PrologueKernArg
         *(u32x4*)(dst + eb * 2) = pack8(x + 8);
       }
     }
+    u = u_next;
+    src = src_n;
+    dst = dst_n;
+    kind = kind_n;
+    va = va_n;
+    vb = vb_n;
   }
 }
 

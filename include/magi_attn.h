@@ -55,7 +55,7 @@ extern "C" {
  * to box); the 32x32x16 form issues half as many MFMAs and is the better one where the clock, not the power, is
  * capped.  512-row workgroups (q_tile_rows) always use it. */
 #define MAGI_ATTN_BOUNDED_MFMA32 8
-/* bf16 without a score_bound: measure one.  Two streaming passes over q and k (256 bytes per (token, head) row: 0.5 ms
+/* bf16 without a score_bound: measure one.  Two streaming passes over q and k (256 bytes per (token, head) row: 0.3 ms
  * at the 720p shape) leave the largest squared row length of each in `workspace`; |q . k| <= |q| |k| for every pair,
  * so the bounded-score kernel and the online-softmax kernel are both launched behind them, each tests
  * max|q| max|k| softmax_scale log2(e) * 1.01 <= MAGI_SCORE_BOUND_MAX on the device, and only the one the test selects

@@ -308,6 +308,9 @@ def test_repeated_launches_are_bit_identical(dev):
     tq, tk = _ranges(dev, O.q_ranges_for(dn, L), O.default_kvrange(sp, dn, L))
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     first, lse0 = M.range_attention(qd, kd, vd, tq, tk, L)
+    bound = 1.01 * (qd.float().norm(dim=-1).max() * kd.float().norm(dim=-1).max()).item() / math.sqrt(128) * math.log2(math.e)
+    assert bound <= M.MAGI_SCORE_BOUND_MAX
+    first_b, lse0_b = M.range_attention(qd, kd, vd, tq, tk, L, score_bound=bound)  # the bounded-score kernel
     q8, qs = M.quantize_fp8(qd, L)
     k8, ks = M.quantize_fp8(kd, L)
     v8, vs = M.quantize_fp8(vd, L)
@@ -315,6 +318,8 @@ def test_repeated_launches_are_bit_identical(dev):
     for _ in range(3):
         noise = torch.randn(1 << 20, device=dev).sum()  # unrelated work in between
         again, lse = M.range_attention(qd, kd, vd, tq, tk, L)
+        again_b, lse_b = M.range_attention(qd, kd, vd, tq, tk, L, score_bound=bound)
+        assert torch.equal(again_b, first_b) and torch.equal(lse_b, lse0_b)
         again8, _ = M.range_attention(q8, k8, v8, tq, tk, L, q_scale=qs, k_scale=ks, v_scale=vs, scale_chunk_tokens=L)
         assert torch.equal(again, first) and torch.equal(lse, lse0) and torch.equal(again8, first8)
         del noise
